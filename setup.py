@@ -42,14 +42,18 @@ class HipBuildExt(build_ext):
     inc = ce.include_paths(device_type="cuda") + [sysconfig.get_paths()["include"], os.path.join(HERE, CSRC)]
     cflags = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-fgpu-flush-denormals-to-zero",
               "-munsafe-fp-atomics", f"-D_GLIBCXX_USE_CXX11_ABI={abi}", "-DTORCH_API_INCLUDE_EXTENSION_H",
-              f"-DTORCH_EXTENSION_NAME={ext.name.split('.')[-1]}", "-DUSE_ROCM=1", "-Wno-unused-result"]
+              f"-DTORCH_EXTENSION_NAME={ext.name.split('.')[-1]}", "-DUSE_ROCM=1", "-Wno-unused-result",
+              # no packed-fp32 VALU forms (v_pk_fma_f32 and friends): plain fp32 code compiles to scalar-lane ops
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     cflags += [f"-I{p}" for p in inc]
     objs, jobs = [], []
+    stamp = os.path.join(tmp, "flags.txt")  # objects built with other flags are stale too
+    flags_same = os.path.exists(stamp) and open(stamp).read() == " ".join(cflags)
     for src in ext.sources:
       obj = os.path.join(tmp, os.path.basename(src) + ".o")
       objs.append(obj)
       deps = [src] + glob.glob(os.path.join(CSRC, "*.h"))
-      if self.force or not os.path.exists(obj) or os.path.getmtime(obj) < max(os.path.getmtime(d) for d in deps):
+      if self.force or not flags_same or not os.path.exists(obj) or os.path.getmtime(obj) < max(os.path.getmtime(d) for d in deps):
         jobs.append([HIPCC, "-c", src, "-o", obj] + cflags)
 
     def run(cmd):
@@ -58,6 +62,8 @@ class HipBuildExt(build_ext):
 
     with ThreadPoolExecutor(max_workers=int(os.environ.get("MAX_JOBS", "8"))) as ex:
       list(ex.map(run, jobs))
+    with open(stamp, "w") as f:
+      f.write(" ".join(cflags))
     libs = ["c10", "torch", "torch_cpu", "torch_python", "c10_hip", "torch_hip", "amdhip64"]
     ldirs = ce.library_paths(device_type="cuda")
     link = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", out] + objs + \

@@ -5,6 +5,10 @@
 #include <ATen/hip/HIPContext.h>
 #include "kernels.h"
 
+namespace xot {
+void bind_mixers(pybind11::module& m);  // csrc/mixers.hip
+}
+
 namespace {
 
 #define XCHECK(cond, ...) TORCH_CHECK(cond, "xot kernel: ", __VA_ARGS__)
@@ -1014,6 +1018,7 @@ void adamw(at::Tensor& p, const at::Tensor& g, at::Tensor& m, at::Tensor& v, con
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "xot MI355X (gfx950) kernel library";
+  xot::bind_mixers(m);
   m.def("rmsnorm", &rmsnorm);
   m.def("rmsnorm_bwd", &rmsnorm_bwd, py::arg("x"), py::arg("w"), py::arg("dy"), py::arg("dx"), py::arg("dw"),
         py::arg("eps"), py::arg("res") = py::none());

@@ -1,0 +1,672 @@
+// Token mixers beside softmax attention, and the fp32-residual layer plumbing around them (gfx950).
+//
+//   resid_scale_norm   x += s1 * y1 (+ s2 * y2) on the fp32 residual stream, then RMS norm with one scalar gain
+//   gelu_mul           gelu_tanh(gate) * up out of a fused projection's columns
+//   rope_kv_store      partial rotate-half RoPE on q and k, paged write of the rotated key and of the value
+//                      (the value may be the un-rotated key)
+//   attn_gated_chunk   chunk-local attention with sigmoid(score + bias[head]) weights, no normalisation
+//   delta_prep         short causal convolutions + SiLU, unit-norm q / k, sigmoid write strength, scalar decay
+//   conv_state_update  the last taps-1 convolution inputs of every sequence -> its state slot
+//   gla_prep           per-key-channel decay sigmoid(low-rank z)^(1/tau)
+//   linear_recurrence  S <- decay * S, delta-rule or outer-product write, o = S^T q; fp32 state per slot
+//   gated_rmsnorm      per-head RMS norm of o, weight, SiLU gate
+//
+// A fused projection's output P is fp32 [T, ldp]; "column offset" arguments address its slices.  Activations that
+// feed the next GEMM (AT) are bf16 or fp32; everything that enters a norm, a score or a recurrence is fp32.
+#include <torch/extension.h>
+#include <ATen/hip/HIPContext.h>
+#include "common.h"
+
+namespace xot {
+namespace {
+
+constexpr int PAGE_TOK = 64;
+
+__device__ __forceinline__ float ldf(const float* p) { return *p; }
+__device__ __forceinline__ float ldf(const uint16_t* p) { return bf2f(*p); }
+__device__ __forceinline__ void stf(float* p, float v) { *p = v; }
+__device__ __forceinline__ void stf(uint16_t* p, float v) { *p = f2bf(v); }
+
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float siluf_(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float softplusf_(float x) { return log1pf(expf(-fabsf(x))) + fmaxf(x, 0.0f); }
+__device__ __forceinline__ float logsigmoidf_(float x) { return fminf(x, 0.0f) - log1pf(expf(-fabsf(x))); }
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  float t = 0.0f;
+  for (int i = 0; i < nw; ++i) t += red[i];
+  return t;
+}
+
+// sequence of token t: the b with cu[b] <= t < cu[b + 1]
+__device__ __forceinline__ int seq_of(const int* cu, int B, int t) {
+  int lo = 0, hi = B - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+// ------------------------------------------------------------------ residual + scalar-gain RMS norm
+template <typename AT>
+__global__ void resid_scale_norm_k(float* __restrict__ x, const float* __restrict__ y1, const float* __restrict__ s1,
+                                   const float* __restrict__ y2, const float* __restrict__ s2,
+                                   const float* __restrict__ gain, float eps, AT* __restrict__ out, int D, int ld1,
+                                   int ld2, int ldo) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  float* xr = x + r * D;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    float v = xr[i];
+    if (y1) {
+      float a = s1[i] * y1[r * ld1 + i];
+      if (y2) a += s2[i] * y2[r * ld2 + i];
+      v += a;
+      xr[i] = v;
+    }
+    ss += v * v;
+  }
+  if (!out) return;
+  ss = block_sum(ss, red);
+  const float k = gain[0] / sqrtf(ss / (float)D + eps);
+  for (int i = threadIdx.x; i < D; i += blockDim.x) stf(out + r * ldo + i, xr[i] * k);
+}
+
+// ------------------------------------------------------------------ gelu_tanh(gate) * up
+template <typename AT>
+__global__ void gelu_mul_k(const float* __restrict__ P, int ldp, int gate_off, int up_off, int F, AT* __restrict__ out,
+                           int ldo, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t t = idx / F;
+  const int i = (int)(idx - t * F);
+  const float z = P[t * ldp + gate_off + i], u = P[t * ldp + up_off + i];
+  const float g = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  stf(out + t * ldo + i, g * u);
+}
+
+// ------------------------------------------------------------------ RoPE + paged key / value write
+// cos_sin [rows, R]: row p = [cos(p f_0 .. f_{R/2-1}) | sin(...)].  Pair (i, i + R/2), i < R/2; dims >= R pass.
+template <typename AT>
+__global__ void rope_kv_store_k(const float* __restrict__ P, int ldp, int q_off, int k_off, int v_off, int H, int G, int d,
+                                int R, const int* __restrict__ pos, const float* __restrict__ cos_sin,
+                                const int64_t* __restrict__ slots, AT* __restrict__ q_out, AT* __restrict__ k_cache,
+                                AT* __restrict__ v_cache) {
+  const int t = blockIdx.x;
+  const float* row = P + (int64_t)t * ldp;
+  const float* cs = cos_sin + (int64_t)pos[t] * R;
+  const int half = R >> 1;
+  const int64_t slot = slots[t];
+  const int n = (H + G) * d;
+  for (int e = threadIdx.x; e < n; e += blockDim.x) {
+    const int head = e / d, i = e - head * d;
+    const bool isq = head < H;
+    const float* x = row + (isq ? q_off + head * d : k_off + (head - H) * d);
+    float v = x[i];
+    const float raw = v;
+    if (i < half) {
+      v = x[i] * cs[i] - x[i + half] * cs[half + i];
+    } else if (i < R) {
+      const int j = i - half;
+      v = x[i] * cs[j] + x[j] * cs[half + j];
+    }
+    if (isq) {
+      stf(q_out + ((int64_t)t * H + head) * d + i, v);
+    } else if (slot >= 0) {
+      const int g = head - H;
+      const int64_t o = (((slot / PAGE_TOK) * G + g) * PAGE_TOK + (slot % PAGE_TOK)) * d + i;
+      stf(k_cache + o, v);
+      stf(v_cache + o, v_off >= 0 ? row[v_off + g * d + i] : raw);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ chunk-local gated attention
+// One wave per (token, head).  Keys of the query's chunk up to the query: lanes over keys for the scores, then lanes
+// over value dims for the weighted sum.  out[t, h * d + i] = out_scale * sum_j sigmoid(q.k_j * scale + pb[h]) v_j[i].
+constexpr int ATT_TILE = 512;
+
+template <typename AT>
+__global__ void attn_gated_chunk_k(const AT* __restrict__ q, const AT* __restrict__ k_cache, const AT* __restrict__ v_cache,
+                                   const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q,
+                                   const int* __restrict__ ctx_lens, int B, const float* __restrict__ pb, float scale,
+                                   int chunk, float out_scale, AT* __restrict__ out, int ldo, int H, int G, int d) {
+  extern __shared__ float sm[];
+  float* qs = sm;            // [d]
+  float* ws = sm + d;        // [ATT_TILE]
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int b = seq_of(cu_q, B, t);
+  const int ctx = ctx_lens[b];
+  if (ctx <= 0) return;  // padding row of a captured decode batch
+  const int pos = ctx - (cu_q[b + 1] - cu_q[b]) + (t - cu_q[b]);
+  const int lo = (pos / chunk) * chunk;
+  const int nkeys = pos - lo + 1;
+  const int g = h / (H / G);
+  for (int i = lane; i < d; i += 64) qs[i] = ldf(q + ((int64_t)t * H + h) * d + i);
+  const float bias = pb[h];
+  const int* bt = block_tables + (int64_t)b * width;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};  // value dims lane, lane + 64, ... (d <= 256)
+  for (int j0 = 0; j0 < nkeys; j0 += ATT_TILE) {
+    const int nj = min(ATT_TILE, nkeys - j0);
+    __syncthreads();
+    for (int j = lane; j < nj; j += 64) {
+      const int p = lo + j0 + j;
+      const AT* kr = k_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * PAGE_TOK + (p % PAGE_TOK)) * d;
+      float s = 0.0f;
+      for (int i = 0; i < d; ++i) s += qs[i] * ldf(kr + i);
+      ws[j] = sigmoidf_(s * scale + bias);
+    }
+    __syncthreads();
+    for (int j = 0; j < nj; ++j) {
+      const int p = lo + j0 + j;
+      const AT* vr = v_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * PAGE_TOK + (p % PAGE_TOK)) * d;
+      const float w = ws[j];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int i = lane + 64 * c;
+        if (i < d) acc[c] += w * ldf(vr + i);
+      }
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int i = lane + 64 * c;
+    if (i < d) stf(out + (int64_t)t * ldo + h * d + i, acc[c] * out_scale);
+  }
+}
+
+// ------------------------------------------------------------------ delta-rule inputs
+// Channels [q: G d | k: G d | v: H dv] at P[:, x_off ...]; conv_w [C, taps] (last column: the current token);
+// conv_state [slots, taps - 1, C] holds the inputs before this step (zeros for a new sequence).
+// qkv [T, C]: q = unit(silu(conv q)) * d^-1/2, k = unit(silu(conv k)), v = silu(conv v);
+// beta [T, H] = sigmoid(P[b_off + h]); decay [T, H] = exp(-exp(A_log[h]) softplus(P[a_off + h] + dt_bias[h])).
+__global__ void delta_prep_k(const float* __restrict__ P, int ldp, int x_off, int b_off, int a_off,
+                             const float* __restrict__ conv_w, int taps, const float* __restrict__ conv_state,
+                             const int* __restrict__ state_slots, const int* __restrict__ cu_q, int B,
+                             const float* __restrict__ A_log, const float* __restrict__ dt_bias, int H, int G, int d, int dv,
+                             float* __restrict__ qkv, float* __restrict__ beta, float* __restrict__ decay) {
+  extern __shared__ float ys[];  // [C]
+  const int t = blockIdx.x;
+  const int b = seq_of(cu_q, B, t);
+  const int slot = state_slots[b];
+  if (slot < 0) return;
+  const int C = 2 * G * d + H * dv;
+  const int local = t - cu_q[b];
+  const float* st = conv_state + (int64_t)slot * (taps - 1) * C;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float y = 0.0f;
+    for (int j = 0; j < taps; ++j) {
+      const int s = local - (taps - 1 - j);
+      const float x = s >= 0 ? P[(int64_t)(cu_q[b] + s) * ldp + x_off + c] : st[(int64_t)(taps - 1 + s) * C + c];
+      y += conv_w[c * taps + j] * x;
+    }
+    ys[c] = siluf_(y);
+  }
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  float* o = qkv + (int64_t)t * C;
+  for (int hd = wave; hd < 2 * G; hd += nw) {  // q heads then k heads
+    const float* y = ys + hd * d;
+    float ss = 0.0f;
+    for (int i = lane; i < d; i += 64) ss += y[i] * y[i];
+    ss = wave_sum(ss);
+    float k = 1.0f / sqrtf(ss + 1e-6f);
+    if (hd < G) k *= 1.0f / sqrtf((float)d);
+    for (int i = lane; i < d; i += 64) o[hd * d + i] = y[i] * k;
+  }
+  for (int c = 2 * G * d + threadIdx.x; c < C; c += blockDim.x) o[c] = ys[c];
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    const float* row = P + (int64_t)t * ldp;
+    beta[(int64_t)t * H + h] = sigmoidf_(row[b_off + h]);
+    decay[(int64_t)t * H + h] = expf(-expf(A_log[h]) * softplusf_(row[a_off + h] + dt_bias[h]));
+  }
+}
+
+__global__ void conv_state_update_k(const float* __restrict__ P, int ldp, int x_off, int C, int taps,
+                                    float* __restrict__ conv_state, const int* __restrict__ state_slots,
+                                    const int* __restrict__ cu_q) {
+  const int b = blockIdx.x;
+  const int slot = state_slots[b];
+  const int n = cu_q[b + 1] - cu_q[b];
+  if (slot < 0 || n <= 0) return;
+  float* st = conv_state + (int64_t)slot * (taps - 1) * C;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
+    // ascending: entry idx takes the old entry idx + n (> idx) or a token of this step
+    for (int idx = 0; idx < taps - 1; ++idx) {
+      const int s = n - (taps - 1) + idx;
+      st[(int64_t)idx * C + c] = s >= 0 ? P[(int64_t)(cu_q[b] + s) * ldp + x_off + c] : st[(int64_t)(idx + n) * C + c];
+    }
+  }
+}
+
+// ------------------------------------------------------------------ GLA decay
+// decay [T, HD] = exp(logsigmoid(z) / tau), z[c] = a2_b[c] + sum_r a2[c, r] P[t, a1_off + r]
+__global__ void gla_prep_k(const float* __restrict__ P, int ldp, int a1_off, int rank, const float* __restrict__ a2,
+                           const float* __restrict__ a2_b, float inv_tau, int HD, float* __restrict__ decay) {
+  extern __shared__ float ys[];  // [rank]
+  const int t = blockIdx.x;
+  for (int r = threadIdx.x; r < rank; r += blockDim.x) ys[r] = P[(int64_t)t * ldp + a1_off + r];
+  __syncthreads();
+  for (int c = threadIdx.x; c < HD; c += blockDim.x) {
+    float z = 0.0f;
+    for (int r = 0; r < rank; ++r) z += a2[(int64_t)c * rank + r] * ys[r];
+    z += a2_b[c];
+    decay[(int64_t)t * HD + c] = expf(logsigmoidf_(z) * inv_tau);
+  }
+}
+
+// ------------------------------------------------------------------ the recurrence
+// Workgroup = (sequence, value head, block of 64 value channels); 256 threads = 64 columns x 4 row groups, the row
+// group in the low lane bits so the two dot products reduce over lanes l ^ 1, l ^ 2.  A thread keeps rows
+// rg + 4 m (m < KR) of its column in registers.  Tokens are staged through LDS REC_TB at a time.
+// DELTA: S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q.   else: S = diag(a) S + k v^T; o = S^T q.
+constexpr int REC_TB = 16;
+
+template <int KR, bool DELTA>
+__global__ __launch_bounds__(256) void linear_recurrence_k(
+    const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
+    const float* __restrict__ decay, const float* __restrict__ beta, float q_scale, float* __restrict__ state,
+    const int* __restrict__ state_slots, const int* __restrict__ cu_q, int H, int G, int d, int dv,
+    float* __restrict__ out) {
+  constexpr int DP = KR * 4;  // padded key dim
+  __shared__ float sq[REC_TB][DP], sk[REC_TB][DP], sa[REC_TB][DELTA ? 1 : DP], sv[REC_TB][64], sg[REC_TB][2];
+  const int b = blockIdx.x, h = blockIdx.y, cb = blockIdx.z;
+  const int slot = state_slots[b];
+  const int t0 = cu_q[b], n = cu_q[b + 1] - t0;
+  if (slot < 0 || n <= 0) return;
+  const int tid = threadIdx.x, rg = tid & 3, col = cb * 64 + (tid >> 2);
+  const bool live = col < dv;
+  const int hk = h / (H / G);
+  float* S = state + (((int64_t)slot * H + h) * d) * dv;
+  float s[KR];
+#pragma unroll
+  for (int m = 0; m < KR; ++m) {
+    const int i = rg + 4 * m;
+    s[m] = (live && i < d) ? S[(int64_t)i * dv + col] : 0.0f;
+  }
+  for (int tb = 0; tb < n; tb += REC_TB) {
+    const int nt = min(REC_TB, n - tb);
+    __syncthreads();
+    for (int e = tid; e < nt * DP; e += 256) {
+      const int tt = e / DP, i = e - tt * DP;
+      const int64_t t = t0 + tb + tt;
+      const bool in = i < d;
+      sq[tt][i] = in ? q[t * ldq + hk * d + i] * q_scale : 0.0f;
+      sk[tt][i] = in ? k[t * ldk + hk * d + i] : 0.0f;
+      if (!DELTA) sa[tt][i] = in ? decay[(t * H + h) * d + i] : 0.0f;
+    }
+    for (int e = tid; e < nt * 64; e += 256) {
+      const int tt = e >> 6, c = cb * 64 + (e & 63);
+      sv[tt][e & 63] = c < dv ? v[(int64_t)(t0 + tb + tt) * ldv + h * dv + c] : 0.0f;
+    }
+    if (DELTA && tid < nt) {
+      sg[tid][0] = decay[(int64_t)(t0 + tb + tid) * H + h];
+      sg[tid][1] = beta[(int64_t)(t0 + tb + tid) * H + h];
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float vc = sv[tt][tid >> 2];
+      float o = 0.0f;
+      if (DELTA) {
+        const float g = sg[tt][0], bt = sg[tt][1];
+        float dot = 0.0f;
+#pragma unroll
+        for (int m = 0; m < KR; ++m) {
+          s[m] *= g;
+          dot += s[m] * sk[tt][rg + 4 * m];
+        }
+        dot += __shfl_xor(dot, 1, 64);
+        dot += __shfl_xor(dot, 2, 64);
+        const float u = bt * (vc - dot);
+#pragma unroll
+        for (int m = 0; m < KR; ++m) {
+          s[m] += sk[tt][rg + 4 * m] * u;
+          o += s[m] * sq[tt][rg + 4 * m];
+        }
+      } else {
+#pragma unroll
+        for (int m = 0; m < KR; ++m) {
+          s[m] = sa[tt][rg + 4 * m] * s[m] + sk[tt][rg + 4 * m] * vc;
+          o += s[m] * sq[tt][rg + 4 * m];
+        }
+      }
+      o += __shfl_xor(o, 1, 64);
+      o += __shfl_xor(o, 2, 64);
+      if (live && rg == 0) out[(int64_t)(t0 + tb + tt) * H * dv + h * dv + col] = o;
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int m = 0; m < KR; ++m) {
+      const int i = rg + 4 * m;
+      if (i < d) S[(int64_t)i * dv + col] = s[m];
+    }
+  }
+}
+
+// ------------------------------------------------------------------ per-head RMS norm * weight * silu(gate)
+template <typename AT>
+__global__ void gated_rmsnorm_k(const float* __restrict__ o, const float* __restrict__ w, const float* __restrict__ P, int ldp,
+                                int g_off, float eps, float out_scale, AT* __restrict__ out, int ldo, int H, int dv) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float* x = o + ((int64_t)t * H + h) * dv;
+  float ss = 0.0f;
+  for (int i = lane; i < dv; i += 64) ss += x[i] * x[i];
+  ss = wave_sum(ss);
+  const float k = out_scale / sqrtf(ss / (float)dv + eps);
+  for (int i = lane; i < dv; i += 64) {
+    const float gate = P[(int64_t)t * ldp + g_off + h * dv + i];
+    stf(out + (int64_t)t * ldo + h * dv + i, x[i] * k * w[i] * siluf_(gate));
+  }
+}
+
+// ------------------------------------------------------------------ host side
+#define MCHECK(cond, ...) TORCH_CHECK(cond, "xot mixers: ", __VA_ARGS__)
+
+inline hipStream_t stream() { return at::hip::getCurrentHIPStream().stream(); }
+inline bool is_act(const at::Tensor& t) { return t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat; }
+inline void f32c(const at::Tensor& t, const char* name) {
+  MCHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), name, " must be a contiguous fp32 GPU tensor");
+}
+inline void i32c(const at::Tensor& t, const char* name) {
+  MCHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), name, " must be a contiguous int32 GPU tensor");
+}
+// fused projection output: fp32 rows of unit inner stride
+inline int ld_of(const at::Tensor& P, const char* name) {
+  MCHECK(P.is_cuda() && P.scalar_type() == at::kFloat && P.dim() == 2 && P.stride(1) == 1, name, " must be fp32 [T, n] rows");
+  return (int)P.stride(0);
+}
+inline void cols_ok(const at::Tensor& P, int64_t off, int64_t n, const char* what) {
+  MCHECK(off >= 0 && n >= 0 && off + n <= P.size(1), what, ": columns [", off, ", ", off + n, ") outside the projection");
+}
+// activation output rows (bf16 / fp32), maybe a column slice of a wider buffer
+inline int act_ld(const at::Tensor& t, int64_t T, int64_t n, const char* name) {
+  MCHECK(t.is_cuda() && is_act(t) && t.dim() == 2 && t.size(0) == T && t.size(1) == n && t.stride(1) == 1, name,
+         " must be [T, ", n, "] bf16 / fp32 rows");
+  return (int)t.stride(0);
+}
+
+void resid_scale_norm(at::Tensor& x, const c10::optional<at::Tensor>& y1, const c10::optional<at::Tensor>& s1,
+                      const c10::optional<at::Tensor>& y2, const c10::optional<at::Tensor>& s2,
+                      const c10::optional<at::Tensor>& gain, double eps, const c10::optional<at::Tensor>& out) {
+  f32c(x, "x");
+  MCHECK(x.dim() == 2, "x must be [T, D]");
+  const int64_t T = x.size(0), D = x.size(1);
+  if (T == 0) return;
+  auto chk = [&](const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& s) {
+    if (!y.has_value()) return;
+    MCHECK(ld_of(*y, "y") >= D && y->size(0) == T && y->size(1) >= D, "residual branch must be fp32 [T, >= D] rows");
+    MCHECK(s.has_value(), "a residual branch needs its scale");
+    f32c(*s, "scale");
+    MCHECK(s->numel() == D, "residual branch scale must hold D numbers");
+  };
+  chk(y1, s1);
+  chk(y2, s2);
+  MCHECK(y1.has_value() || !y2.has_value(), "y2 without y1");
+  if (out.has_value()) {
+    MCHECK(gain.has_value(), "a normed output needs the gain");
+    f32c(*gain, "gain");
+    MCHECK(gain->numel() == 1, "gain must hold one number");
+    MCHECK(out->is_cuda() && is_act(*out) && out->dim() == 2 && out->size(0) == T && out->size(1) >= D && out->stride(1) == 1,
+           "out must be [T, >= D] rows");
+  }
+  const int ld1 = y1.has_value() ? (int)y1->stride(0) : 0, ld2 = y2.has_value() ? (int)y2->stride(0) : 0;
+  const int ldo = out.has_value() ? (int)out->stride(0) : 0;
+  const float* p1 = y1.has_value() ? y1->data_ptr<float>() : nullptr;
+  const float* q1 = y1.has_value() ? s1->data_ptr<float>() : nullptr;
+  const float* p2 = y2.has_value() ? y2->data_ptr<float>() : nullptr;
+  const float* q2 = y2.has_value() ? s2->data_ptr<float>() : nullptr;
+  const float* g = out.has_value() ? gain->data_ptr<float>() : nullptr;
+  if (out.has_value() && out->scalar_type() == at::kBFloat16)
+    resid_scale_norm_k<uint16_t><<<T, 256, 0, stream()>>>(x.data_ptr<float>(), p1, q1, p2, q2, g, (float)eps,
+                                                          (uint16_t*)out->data_ptr(), (int)D, ld1, ld2, ldo);
+  else
+    resid_scale_norm_k<float><<<T, 256, 0, stream()>>>(x.data_ptr<float>(), p1, q1, p2, q2, g, (float)eps,
+                                                       out.has_value() ? out->data_ptr<float>() : nullptr, (int)D, ld1, ld2, ldo);
+}
+
+void gelu_mul(const at::Tensor& P, int64_t gate_off, int64_t up_off, int64_t F, at::Tensor& out) {
+  const int ldp = ld_of(P, "P");
+  const int64_t T = P.size(0);
+  MCHECK(out.is_cuda() && is_act(out) && out.dim() == 2 && out.size(0) == T && out.size(1) >= F && out.stride(1) == 1,
+         "out must be [T, >= F] rows");
+  const int ldo = (int)out.stride(0);
+  cols_ok(P, gate_off, F, "gate");
+  cols_ok(P, up_off, F, "up");
+  const int64_t total = T * F;
+  if (total == 0) return;
+  const int blocks = (int)((total + 255) / 256);
+  if (out.scalar_type() == at::kBFloat16)
+    gelu_mul_k<uint16_t><<<blocks, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)gate_off, (int)up_off, (int)F,
+                                                       (uint16_t*)out.data_ptr(), ldo, total);
+  else
+    gelu_mul_k<float><<<blocks, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)gate_off, (int)up_off, (int)F,
+                                                    out.data_ptr<float>(), ldo, total);
+}
+
+void rope_kv_store(const at::Tensor& P, int64_t q_off, int64_t k_off, int64_t v_off, int64_t H, int64_t G, int64_t d,
+                   int64_t R, const at::Tensor& pos, const at::Tensor& cos_sin, const at::Tensor& slots, at::Tensor& q_out,
+                   at::Tensor& k_cache, at::Tensor& v_cache) {
+  const int ldp = ld_of(P, "P");
+  const int64_t T = P.size(0);
+  if (T == 0) return;
+  i32c(pos, "pos");
+  f32c(cos_sin, "cos_sin");
+  MCHECK(slots.is_cuda() && slots.scalar_type() == at::kLong && slots.is_contiguous() && slots.numel() == T && pos.numel() == T,
+         "pos / slots must hold one entry per token");
+  MCHECK(R % 2 == 0 && R >= 0 && R <= d && (R == 0 || (cos_sin.dim() == 2 && cos_sin.size(1) == R)), "bad rotary dims");
+  cols_ok(P, q_off, H * d, "q");
+  cols_ok(P, k_off, G * d, "k");
+  if (v_off >= 0) cols_ok(P, v_off, G * d, "v");
+  MCHECK(q_out.is_cuda() && is_act(q_out) && q_out.is_contiguous() && q_out.numel() == T * H * d, "q_out must be [T, H, d]");
+  MCHECK(k_cache.is_cuda() && k_cache.scalar_type() == q_out.scalar_type() && k_cache.is_contiguous() && k_cache.dim() == 4 &&
+             k_cache.size(1) == G && k_cache.size(2) == PAGE_TOK && k_cache.size(3) == d,
+         "k_cache must be [pages, G, 64, d] of q_out's dtype");
+  MCHECK(v_cache.is_cuda() && v_cache.scalar_type() == q_out.scalar_type() && v_cache.is_contiguous() &&
+             v_cache.sizes() == k_cache.sizes(), "v_cache must match k_cache");
+  // positions and slots are checked on the host by their producer (the block manager hands out slots < pages * 64
+  // and the runner bounds positions by the table's rows)
+  if (q_out.scalar_type() == at::kBFloat16)
+    rope_kv_store_k<uint16_t><<<T, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)q_off, (int)k_off, (int)v_off, (int)H,
+                                                       (int)G, (int)d, (int)R, pos.data_ptr<int>(), cos_sin.data_ptr<float>(),
+                                                       slots.data_ptr<int64_t>(), (uint16_t*)q_out.data_ptr(),
+                                                       (uint16_t*)k_cache.data_ptr(), (uint16_t*)v_cache.data_ptr());
+  else
+    rope_kv_store_k<float><<<T, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)q_off, (int)k_off, (int)v_off, (int)H, (int)G,
+                                                    (int)d, (int)R, pos.data_ptr<int>(), cos_sin.data_ptr<float>(),
+                                                    slots.data_ptr<int64_t>(), q_out.data_ptr<float>(),
+                                                    k_cache.data_ptr<float>(), v_cache.data_ptr<float>());
+}
+
+void attn_gated_chunk(const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache, const at::Tensor& block_tables,
+                      const at::Tensor& cu_q, const at::Tensor& ctx_lens, const at::Tensor& pb, double scale, int64_t chunk,
+                      double out_scale, at::Tensor& out) {
+  MCHECK(q.is_cuda() && is_act(q) && q.is_contiguous() && q.dim() == 3, "q must be [T, H, d]");
+  const int64_t T = q.size(0), H = q.size(1), d = q.size(2);
+  if (T == 0) return;
+  MCHECK(k_cache.is_cuda() && k_cache.scalar_type() == q.scalar_type() && k_cache.is_contiguous() && k_cache.dim() == 4 &&
+             k_cache.size(2) == PAGE_TOK && k_cache.size(3) == d, "k_cache must be [pages, G, 64, d] of q's dtype");
+  MCHECK(v_cache.is_cuda() && v_cache.scalar_type() == q.scalar_type() && v_cache.is_contiguous() &&
+             v_cache.sizes() == k_cache.sizes(), "v_cache must match k_cache");
+  const int64_t G = k_cache.size(1);
+  MCHECK(G > 0 && H % G == 0 && d <= 256 && chunk > 0, "attn_gated_chunk: heads must be a multiple of kv heads, d <= 256");
+  i32c(block_tables, "block_tables");
+  i32c(cu_q, "cu_q");
+  i32c(ctx_lens, "ctx_lens");
+  f32c(pb, "pb");
+  const int64_t B = ctx_lens.numel();
+  MCHECK(block_tables.dim() == 2 && block_tables.size(0) == B && cu_q.numel() == B + 1 && pb.numel() == H, "batch shape mismatch");
+  const int ldo = act_ld(out, T, H * d, "out");
+  MCHECK(out.scalar_type() == q.scalar_type(), "out must have q's dtype");
+  const dim3 grid((unsigned)T, (unsigned)H);
+  const size_t lds = (d + ATT_TILE) * sizeof(float);
+  if (q.scalar_type() == at::kBFloat16)
+    attn_gated_chunk_k<uint16_t><<<grid, 64, lds, stream()>>>(
+        (const uint16_t*)q.data_ptr(), (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(),
+        block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B,
+        pb.data_ptr<float>(), (float)scale, (int)chunk, (float)out_scale, (uint16_t*)out.data_ptr(), ldo, (int)H, (int)G, (int)d);
+  else
+    attn_gated_chunk_k<float><<<grid, 64, lds, stream()>>>(
+        q.data_ptr<float>(), k_cache.data_ptr<float>(), v_cache.data_ptr<float>(), block_tables.data_ptr<int>(),
+        (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, pb.data_ptr<float>(), (float)scale,
+        (int)chunk, (float)out_scale, out.data_ptr<float>(), ldo, (int)H, (int)G, (int)d);
+}
+
+void delta_prep(const at::Tensor& P, int64_t x_off, int64_t b_off, int64_t a_off, const at::Tensor& conv_w,
+                at::Tensor& conv_state, const at::Tensor& state_slots, const at::Tensor& cu_q, const at::Tensor& A_log,
+                const at::Tensor& dt_bias, int64_t H, int64_t G, int64_t d, int64_t dv, at::Tensor& qkv, at::Tensor& beta,
+                at::Tensor& decay) {
+  const int ldp = ld_of(P, "P");
+  const int64_t T = P.size(0), C = 2 * G * d + H * dv;
+  if (T == 0) return;
+  f32c(conv_w, "conv_w");
+  f32c(conv_state, "conv_state");
+  f32c(A_log, "A_log");
+  f32c(dt_bias, "dt_bias");
+  f32c(qkv, "qkv");
+  f32c(beta, "beta");
+  f32c(decay, "decay");
+  i32c(state_slots, "state_slots");
+  i32c(cu_q, "cu_q");
+  MCHECK(conv_w.dim() == 2 && conv_w.size(0) == C, "conv_w must be [C, taps]");
+  const int64_t taps = conv_w.size(1), B = state_slots.numel();
+  MCHECK(taps >= 1 && conv_state.dim() == 3 && conv_state.size(1) == taps - 1 && conv_state.size(2) == C,
+         "conv_state must be [slots, taps - 1, C]");
+  MCHECK(cu_q.numel() == B + 1 && A_log.numel() == H && dt_bias.numel() == H && H % G == 0, "delta_prep: shape mismatch");
+  MCHECK(qkv.numel() == T * C && beta.numel() == T * H && decay.numel() == T * H, "delta_prep: output shape mismatch");
+  cols_ok(P, x_off, C, "conv inputs");
+  cols_ok(P, b_off, H, "beta");
+  cols_ok(P, a_off, H, "decay");
+  MCHECK(C * sizeof(float) <= 64 * 1024, "delta_prep: too many convolution channels");
+  delta_prep_k<<<T, 256, C * sizeof(float), stream()>>>(
+      P.data_ptr<float>(), ldp, (int)x_off, (int)b_off, (int)a_off, conv_w.data_ptr<float>(), (int)taps,
+      conv_state.data_ptr<float>(), state_slots.data_ptr<int>(), cu_q.data_ptr<int>(), (int)B, A_log.data_ptr<float>(),
+      dt_bias.data_ptr<float>(), (int)H, (int)G, (int)d, (int)dv, qkv.data_ptr<float>(), beta.data_ptr<float>(),
+      decay.data_ptr<float>());
+  if (taps > 1) {
+    const dim3 grid((unsigned)B, (unsigned)((C + 255) / 256));
+    conv_state_update_k<<<grid, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)x_off, (int)C, (int)taps,
+                                                    conv_state.data_ptr<float>(), state_slots.data_ptr<int>(),
+                                                    cu_q.data_ptr<int>());
+  }
+}
+
+void gla_prep(const at::Tensor& P, int64_t a1_off, const at::Tensor& a2, const at::Tensor& a2_b, double tau, at::Tensor& decay) {
+  const int ldp = ld_of(P, "P");
+  const int64_t T = P.size(0);
+  if (T == 0) return;
+  f32c(a2, "a2");
+  f32c(a2_b, "a2_b");
+  f32c(decay, "decay");
+  MCHECK(a2.dim() == 2, "a2 must be [H d, rank]");
+  const int64_t HD = a2.size(0), rank = a2.size(1);
+  MCHECK(a2_b.numel() == HD && decay.numel() == T * HD && tau > 0, "gla_prep: shape mismatch");
+  cols_ok(P, a1_off, rank, "decay projection");
+  gla_prep_k<<<T, 256, rank * sizeof(float), stream()>>>(P.data_ptr<float>(), ldp, (int)a1_off, (int)rank, a2.data_ptr<float>(),
+                                                         a2_b.data_ptr<float>(), (float)(1.0 / tau), (int)HD,
+                                                         decay.data_ptr<float>());
+}
+
+template <bool DELTA>
+void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* decay,
+                const float* beta, float q_scale, float* state, const int* slots, const int* cu, int H, int G, int d, int dv,
+                float* out) {
+#define REC_CASE(N)                                                                                                      \
+  case N:                                                                                                                \
+    linear_recurrence_k<N, DELTA><<<grid, 256, 0, stream()>>>(q, ldq, k, ldk, v, ldv, decay, beta, q_scale, state, slots, \
+                                                              cu, H, G, d, dv, out);                                     \
+    break;
+  switch (KR) {
+    REC_CASE(4)
+    REC_CASE(8)
+    REC_CASE(16)
+    REC_CASE(32)
+    REC_CASE(64)
+    default:
+      MCHECK(false, "linear_recurrence: key dim above 256");
+  }
+#undef REC_CASE
+}
+
+// q / k [T, G d], v [T, H dv]: fp32 rows of unit inner stride (column slices allowed).  decay [T, H] (delta) or
+// [T, H d] (per key channel); beta [T, H] (delta only).  state [slots, H, d, dv].
+void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& decay,
+                       const c10::optional<at::Tensor>& beta, double q_scale, at::Tensor& state, const at::Tensor& state_slots,
+                       const at::Tensor& cu_q, at::Tensor& out) {
+  const int ldq = ld_of(q, "q"), ldk = ld_of(k, "k"), ldv = ld_of(v, "v");
+  f32c(decay, "decay");
+  f32c(state, "state");
+  f32c(out, "out");
+  i32c(state_slots, "state_slots");
+  i32c(cu_q, "cu_q");
+  MCHECK(state.dim() == 4, "state must be [slots, H, d, dv]");
+  const int64_t T = q.size(0), H = state.size(1), d = state.size(2), dv = state.size(3), B = state_slots.numel();
+  if (T == 0 || B == 0) return;
+  MCHECK(q.size(1) % d == 0 && q.size(1) == k.size(1), "q / k must be [T, G d]");
+  const int64_t G = q.size(1) / d;
+  MCHECK(G > 0 && H % G == 0 && k.size(0) == T && v.size(0) == T && v.size(1) == H * dv && out.numel() == T * H * dv,
+         "linear_recurrence: shape mismatch");
+  MCHECK(cu_q.numel() == B + 1, "cu_q must hold B + 1 offsets");
+  const bool delta = beta.has_value();
+  if (delta) {
+    f32c(*beta, "beta");
+    MCHECK(beta->numel() == T * H && decay.numel() == T * H, "delta rule: beta / decay must be [T, H]");
+  } else {
+    MCHECK(decay.numel() == T * H * d && G == H, "per-channel decay must be [T, H d] with one q / k head per value head");
+  }
+  int KR = 4;
+  while (KR * 4 < d) KR *= 2;
+  const dim3 grid((unsigned)B, (unsigned)H, (unsigned)((dv + 63) / 64));
+  if (delta)
+    launch_rec<true>(KR, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,
+                     decay.data_ptr<float>(), beta->data_ptr<float>(), (float)q_scale, state.data_ptr<float>(),
+                     state_slots.data_ptr<int>(), cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, out.data_ptr<float>());
+  else
+    launch_rec<false>(KR, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,
+                      decay.data_ptr<float>(), nullptr, (float)q_scale, state.data_ptr<float>(), state_slots.data_ptr<int>(),
+                      cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, out.data_ptr<float>());
+}
+
+void gated_rmsnorm(const at::Tensor& o, const at::Tensor& w, const at::Tensor& P, int64_t g_off, double eps, double out_scale,
+                   at::Tensor& out) {
+  f32c(o, "o");
+  f32c(w, "w");
+  const int ldp = ld_of(P, "P");
+  const int64_t T = P.size(0), dv = w.numel();
+  if (T == 0) return;
+  MCHECK(dv > 0 && o.numel() % (T * dv) == 0, "o must be [T, H, dv]");
+  const int64_t H = o.numel() / (T * dv);
+  cols_ok(P, g_off, H * dv, "gate");
+  const int ldo = act_ld(out, T, H * dv, "out");
+  const dim3 grid((unsigned)T, (unsigned)H);
+  if (out.scalar_type() == at::kBFloat16)
+    gated_rmsnorm_k<uint16_t><<<grid, 64, 0, stream()>>>(o.data_ptr<float>(), w.data_ptr<float>(), P.data_ptr<float>(), ldp,
+                                                         (int)g_off, (float)eps, (float)out_scale, (uint16_t*)out.data_ptr(),
+                                                         ldo, (int)H, (int)dv);
+  else
+    gated_rmsnorm_k<float><<<grid, 64, 0, stream()>>>(o.data_ptr<float>(), w.data_ptr<float>(), P.data_ptr<float>(), ldp,
+                                                      (int)g_off, (float)eps, (float)out_scale, out.data_ptr<float>(), ldo,
+                                                      (int)H, (int)dv);
+}
+
+}  // namespace
+
+void bind_mixers(pybind11::module& m) {
+  m.def("resid_scale_norm", &resid_scale_norm);
+  m.def("gelu_mul", &gelu_mul);
+  m.def("rope_kv_store", &rope_kv_store);
+  m.def("attn_gated_chunk", &attn_gated_chunk);
+  m.def("delta_prep", &delta_prep);
+  m.def("gla_prep", &gla_prep);
+  m.def("linear_recurrence", &linear_recurrence);
+  m.def("gated_rmsnorm", &gated_rmsnorm);
+}
+
+}  // namespace xot

@@ -14,8 +14,55 @@ from typing import Optional
 
 
 @dataclass(frozen=True)
+class GatedAttnSpec:
+  """Chunk-local gated attention: GQA, rotate-half RoPE on the first rot_dims dims of each head, a key is
+  visible to a query of the same chunk-sized block at or before it, and weighs sigmoid(score * scale + bias[head])
+  (no normalisation over keys).  values_are_keys: the value of a token is its key before rotation (no v
+  projection; vdim == dim)."""
+  heads: int
+  kv_heads: int
+  dim: int
+  vdim: int
+  chunk: int
+  rot_dims: int
+  rot_base: float
+  scale: float
+  values_are_keys: bool = True
+
+
+@dataclass(frozen=True)
+class LinearRecurrenceSpec:
+  """A linear-attention state S [dim, vdim] per head carried in fp32: S <- decay * S (+ delta-rule or plain
+  outer-product write), o = S^T q.
+  rule "delta": scalar decay per head g = exp(-exp(A_log) softplus(a + dt_bias)), write k (beta (v - S^T k))^T,
+    q / k shared by heads / kv_heads value heads, short causal convolutions (conv taps) + SiLU on q, k, v,
+    unit-norm q and k, q scaled by dim^-1/2.
+  rule "gla": decay per key channel sigmoid(z)^(1/tau) with a low-rank z, write k v^T, q scaled by dim^-1/2."""
+  rule: str  # delta | gla
+  heads: int
+  kv_heads: int
+  dim: int
+  vdim: int
+  conv: int = 0  # taps of the short convolutions (delta)
+  tau: float = 1.0  # decay temperature (gla)
+  rank: int = 0  # rank of the decay projection (gla; from the tensor's shape)
+
+
+@dataclass(frozen=True)
+class MixedLayerSpec:
+  """One layer of a model whose layers differ (ModelConfig.layer_specs): the token mixers that read the layer's
+  one normed input side by side, their output scales, and the gated feed-forward size (0: none)."""
+  kind: str  # config.json's layer type
+  attn: Optional[GatedAttnSpec] = None
+  rec: Optional[LinearRecurrenceSpec] = None
+  attn_scale: float = 1.0
+  rec_scale: float = 1.0
+  ff: int = 0
+
+
+@dataclass(frozen=True)
 class ModelConfig:
-  model_type: str  # llama | qwen2 | mistral | mixtral
+  model_type: str  # llama | qwen2 | mistral | mixtral | tarepel
   vocab_size: int
   hidden_size: int
   intermediate_size: int
@@ -59,6 +106,19 @@ class ModelConfig:
   vision_feature_layer: int = -2
   vision_select: str = "default"  # default: drop the CLS feature | full
   projector_act: str = "gelu"
+  # models with per-layer mixers (Tarepel): one MixedLayerSpec per layer; parallel mixer + feed-forward blocks on
+  # an fp32 residual stream, scalar-gain RMS norms, per-channel layer scales, scaled logits
+  layer_specs: Optional[tuple] = None
+  logit_scale: float = 1.0
+
+  @property
+  def is_mixed(self) -> bool:
+    return self.layer_specs is not None
+
+  @property
+  def has_state(self) -> bool:
+    """Some layer carries recurrent state per request (a state slot beside the KV pages)."""
+    return bool(self.layer_specs) and any(s.rec is not None for s in self.layer_specs)
 
   @property
   def qkv_size(self) -> int:
@@ -111,6 +171,9 @@ class ModelConfig:
 
   def params_per_layer(self, i: int = -1) -> int:
     D, F = self.hidden_size, self.intermediate_size
+    if self.layer_specs:
+      return sum(mixed_layer_params(D, s) for s in self.layer_specs) // len(self.layer_specs) if i < 0 else \
+        mixed_layer_params(D, self.layer_specs[i])
     if self.is_mla:
       H, dn, dr, dv = self.num_heads, self.qk_nope_head_dim, self.qk_rope_head_dim, self.v_head_dim
       attn = D * self.qkv_size + (self.q_lora_rank * H * (dn + dr) if self.q_lora_rank else 0)
@@ -136,7 +199,25 @@ class ModelConfig:
     return d
 
   def with_layers(self, n: int) -> "ModelConfig":
+    if self.layer_specs is not None and n != len(self.layer_specs):
+      specs = tuple(self.layer_specs[i % len(self.layer_specs)] for i in range(n))
+      return replace(self, num_layers=n, layer_specs=specs)
     return replace(self, num_layers=n)
+
+
+def mixed_layer_params(D: int, s: MixedLayerSpec) -> int:
+  n = 1 + 2 * D + 3 * D * s.ff
+  if s.attn is not None:
+    a = s.attn
+    n += D * a.dim * (a.heads + a.kv_heads * (1 if a.values_are_keys else 2)) + a.heads * a.vdim * D + a.heads
+  if s.rec is not None:
+    r = s.rec
+    n += D * (2 * r.kv_heads * r.dim + 2 * r.heads * r.vdim) + r.heads * r.vdim * D + r.vdim
+    if r.rule == "delta":
+      n += r.conv * (2 * r.kv_heads * r.dim + r.heads * r.vdim) + 2 * r.heads * D + 2 * r.heads
+    else:
+      n += r.rank * (D + r.heads * r.dim) + r.heads * r.dim
+  return n
 
 
 def _rope_fields(cfg: dict) -> tuple:
@@ -164,7 +245,46 @@ def _rope_fields(cfg: dict) -> tuple:
   return theta, (scaling or None), partial
 
 
+def _tarepel_config(cfg: dict) -> ModelConfig:
+  """Tarepel config.json: {"architecture", "vocab", "width", "norm": {"eps"}, "logit_scale", "layers": [{"type":
+  "parallel" | "gla", "mixer": {...}, "mlp": {"kind": "dense", "ff"} | null}]}.  A "parallel" mixer holds a
+  chunked gated attention ("left") beside a gated delta rule ("right") with their output scales; a "gla" mixer
+  is one gated linear attention (its decay rank comes from the checkpoint, see models.weights)."""
+  specs = []
+  for i, L in enumerate(cfg["layers"]):
+    m, mlp = L["mixer"], L.get("mlp")
+    if mlp is not None and mlp.get("kind", "dense") != "dense":
+      raise ValueError(f"layer {i}: unsupported feed-forward kind {mlp.get('kind')!r}")
+    ff = int(mlp["ff"]) if mlp is not None else 0
+    if L["type"] == "parallel":
+      a, r = m["left"], m["right"]
+      if int(a["vdim"]) != int(a["dim"]):
+        raise ValueError(f"layer {i}: values are the keys, so vdim must equal dim")
+      attn = GatedAttnSpec(int(a["heads"]), int(a["kv_heads"]), int(a["dim"]), int(a["vdim"]), int(a["mask"]["size"]),
+                           int(a["rot"]["dims"]), float(a["rot"]["base"]), float(a["scale"]))
+      rec = LinearRecurrenceSpec("delta", int(r["heads"]), int(r["kv_heads"]), int(r["dim"]), int(r["vdim"]),
+                                 conv=int(r["conv"]))
+      specs.append(MixedLayerSpec("parallel", attn, rec, float(m["left_scale"]), float(m["right_scale"]), ff))
+    elif L["type"] == "gla":
+      rec = LinearRecurrenceSpec("gla", int(m["heads"]), int(m["heads"]), int(m["dim"]), int(m["vdim"]),
+                                 tau=float(m["tau"]), rank=int(m.get("rank", 0)))
+      specs.append(MixedLayerSpec("gla", None, rec, 1.0, 1.0, ff))
+    else:
+      raise ValueError(f"layer {i}: unknown layer type {L['type']!r}")
+  first = next((s.attn for s in specs if s.attn is not None), None)
+  return ModelConfig(
+    model_type="tarepel", vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]),
+    intermediate_size=max([s.ff for s in specs] + [0]), num_layers=len(specs),
+    num_heads=first.heads if first else 1, num_kv_heads=first.kv_heads if first else 1,
+    head_dim=first.dim if first else 64, rms_norm_eps=float(cfg["norm"]["eps"]),
+    rope_theta=first.rot_base if first else 10000.0, max_position_embeddings=int(cfg.get("max_positions", 1 << 20)),
+    bos_token_id=int(cfg.get("bos_token_id", 0)), eos_token_ids=tuple(cfg.get("eos_token_ids", ())),
+    layer_specs=tuple(specs), logit_scale=float(cfg.get("logit_scale", 1.0)))
+
+
 def from_hf_config(cfg: dict) -> ModelConfig:
+  if cfg.get("architecture") == "Tarepel":
+    return _tarepel_config(cfg)
   mt = cfg.get("model_type", "llama")
   if mt == "llava":
     return _llava_config(cfg)

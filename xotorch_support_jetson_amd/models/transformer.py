@@ -74,6 +74,8 @@ class StepInputs:
   max_qlen: int
   decode: bool  # every sequence has exactly one new token
   image_embeds: Optional[torch.Tensor] = None  # LLaVA: [n image-token rows, D], in token order (first shard)
+  # models with recurrent layers: [B] int32 state slot of each sequence (-1: padding row, nothing is read or written)
+  state_slots: Optional[torch.Tensor] = None
 
   @property
   def num_tokens(self) -> int:
@@ -89,8 +91,19 @@ class KVCache:
   [8 chunks][Dh][8 keys], ops/reference.py v_chunks).
   MLA models (DeepSeek) keep one latent row per token instead: k = C [L, pages, 64, kv_lora + rope], v None."""
 
-  def __init__(self, c: ModelConfig, n_layers: int, num_pages: int, device, dtype=torch.bfloat16):
+  def __init__(self, c: ModelConfig, n_layers: int, num_pages: int, device, dtype=torch.bfloat16, layer_ids=None):
     self.num_pages = num_pages
+    self.device = torch.device(device)
+    if c.is_mixed:
+      # one K and one V pool per layer that has an attention mixer (None for the others), both [pages, G, 64, d]:
+      # layers may differ in heads and sizes; the value pool holds whatever the layer's mixer stores as values
+      ids = list(layer_ids) if layer_ids is not None else list(range(n_layers))
+      specs = [c.layer_specs[i].attn for i in ids]
+      self.k = [None if a is None else torch.zeros(num_pages, a.kv_heads, PAGE, a.dim, device=device, dtype=dtype)
+                for a in specs]
+      self.v = [None if a is None else torch.zeros(num_pages, a.kv_heads, PAGE, a.dim, device=device, dtype=dtype)
+                for a in specs]
+      return
     if c.is_mla:
       self.k = torch.zeros(n_layers, num_pages, PAGE, c.mla_dim, device=device, dtype=dtype)
       self.v = None
@@ -99,13 +112,42 @@ class KVCache:
     self.v = torch.zeros(n_layers, num_pages, c.num_kv_heads, c.head_dim, PAGE, device=device, dtype=dtype)
 
   @staticmethod
-  def bytes_per_page(c: ModelConfig, n_layers: int) -> int:
+  def bytes_per_page(c: ModelConfig, n_layers: int, layer_ids=None, itemsize: int = 2) -> int:
+    if c.is_mixed:
+      ids = list(layer_ids) if layer_ids is not None else list(range(n_layers))
+      return max(1, sum(2 * a.kv_heads * PAGE * a.dim * itemsize for a in (c.layer_specs[i].attn for i in ids)
+                        if a is not None))
     if c.is_mla:
       return n_layers * PAGE * c.mla_dim * 2
     return 2 * n_layers * c.num_kv_heads * PAGE * c.head_dim * 2
 
   def nbytes(self) -> int:
-    return sum(t.numel() * t.element_size() for t in (self.k, self.v) if t is not None)
+    ts = (self.k + self.v) if isinstance(self.k, list) else (self.k, self.v)
+    return sum(t.numel() * t.element_size() for t in ts if t is not None)
+
+
+class StatePool:
+  """Recurrent state of a shard's layers, one slot per live request (models.config.LinearRecurrenceSpec): per layer
+  with a recurrence S [slots, H, d, dv] fp32 and, for rules with short convolutions, the last taps - 1 convolution
+  inputs [slots, taps - 1, channels] fp32.  A slot is cleared when a request is admitted to it."""
+
+  def __init__(self, c: ModelConfig, layer_ids, slots: int, device):
+    self.slots = slots
+    self.S: List[Optional[torch.Tensor]] = []
+    self.conv: List[Optional[torch.Tensor]] = []
+    for i in layer_ids:
+      r = c.layer_specs[i].rec
+      self.S.append(None if r is None else torch.zeros(slots, r.heads, r.dim, r.vdim, device=device, dtype=torch.float32))
+      ch = 0 if r is None or r.conv <= 0 else 2 * r.kv_heads * r.dim + r.heads * r.vdim
+      self.conv.append(torch.zeros(slots, max(r.conv - 1, 0), ch, device=device, dtype=torch.float32) if ch else None)
+
+  def clear(self, slot: int) -> None:
+    for t in self.S + self.conv:
+      if t is not None:
+        t[slot].zero_()
+
+  def nbytes(self) -> int:
+    return sum(t.numel() * 4 for t in self.S + self.conv if t is not None)
 
 
 class ShardModel:
@@ -114,8 +156,22 @@ class ShardModel:
     self.c: ModelConfig = weights.config
     self.shard: Shard = weights.shard
     self.kv = kv
-    self.device = kv.k.device
+    self.device = kv.device if hasattr(kv, "device") else kv.k.device
     c = self.c
+    self.state: Optional[StatePool] = None  # set by the runner for models with recurrent layers
+    if c.is_mixed:
+      self.layer_ids = list(self.shard.layers())
+      self.max_batch, self.max_ctx, self.ws = max_batch, max_ctx, None
+      self.rope_rows, self.rope_window = max(max_ctx, 16), None
+      self.head_rows, self._head_cache = None, None
+      # one [rows, R] (cos | sin) table per distinct (rotary dims, base) among the attention mixers
+      self.rope_tabs = {}
+      for i in self.layer_ids:
+        a = c.layer_specs[i].attn
+        if a is not None and a.rot_dims and (a.rot_dims, a.rot_base) not in self.rope_tabs:
+          from ..ops.rope import build_cos_sin
+          self.rope_tabs[(a.rot_dims, a.rot_base)] = build_cos_sin(a.rot_dims, self.rope_rows, a.rot_base, None, self.device)
+      return
     self.scale = 1.0 / math.sqrt(c.head_dim)
     max_pos = max(max_ctx, 16)
     self.cos_sin = rope_table(c, max_pos, self.device)
@@ -320,12 +376,118 @@ class ShardModel:
     C.moe_combine(y, slot_of, topw, h, S)
     return None
 
+  # ------------------------------------------------------------------ layers of differing mixers
+  @staticmethod
+  def _proj(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """fp32 x @ w^T: the kernel library's bf16 GEMMs (fp32 accumulate and output), or the vendor SGEMM for an
+    all-fp32 run."""
+    if x.dtype == torch.float32:
+      return torch.matmul(x, w.t())
+    return linear(x, w, out_dtype=torch.float32)
+
+  def _gated_attn(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:
+    """Chunk-local sigmoid attention: RoPE + paged write of (rotated key, key as projected), then the gated sum
+    over the query's chunk, scaled into the mixers' output row."""
+    a = lw.spec.attn
+    q = torch.empty(P.shape[0], a.heads, a.dim, dtype=mix.dtype, device=P.device)
+    tab = self.rope_tabs.get((a.rot_dims, a.rot_base))
+    K.rope_kv_store(P, lw.cols["aq"][0], lw.cols["ak"][0], -1 if a.values_are_keys else lw.cols["av"][0], a.heads,
+                    a.kv_heads, a.dim, a.rot_dims if tab is not None else 0,
+                    inp.positions, tab if tab is not None else torch.zeros(1, 0, device=P.device), inp.slots, q,
+                    self.kv.k[j], self.kv.v[j])
+    off, n = lw.mix_cols["attn"]
+    K.attn_gated_chunk(q, self.kv.k[j], self.kv.v[j], inp.block_tables, inp.cu_q, inp.ctx_lens, lw.attn_pb, a.scale,
+                       a.chunk, lw.spec.attn_scale, mix[:, off:off + n])
+
+  def _recurrence(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:
+    """Linear-attention recurrence over each sequence's state slot (delta rule or per-channel decay), then the
+    per-head gated RMS norm, scaled into the mixers' output row."""
+    r, st, dev = lw.spec.rec, self.state, P.device
+    T = P.shape[0]
+    H, G, d, dv = r.heads, r.kv_heads, r.dim, r.vdim
+    o = torch.empty(T, H * dv, dtype=torch.float32, device=dev)
+    if r.rule == "delta":
+      C = 2 * G * d + H * dv
+      qkv = torch.empty(T, C, dtype=torch.float32, device=dev)
+      beta = torch.empty(T, H, dtype=torch.float32, device=dev)
+      decay = torch.empty(T, H, dtype=torch.float32, device=dev)
+      K.delta_prep(P, lw.cols["rq"][0], lw.cols["rb"][0], lw.cols["ra"][0], lw.conv_w, st.conv[j], inp.state_slots,
+                   inp.cu_q, lw.A_log, lw.dt_bias, H, G, d, dv, qkv, beta, decay)
+      K.linear_recurrence(qkv[:, :G * d], qkv[:, G * d:2 * G * d], qkv[:, 2 * G * d:], decay, beta, 1.0, st.S[j],
+                          inp.state_slots, inp.cu_q, o)
+    else:
+      decay = torch.empty(T, H * d, dtype=torch.float32, device=dev)
+      K.gla_prep(P, lw.cols["ra1"][0], lw.a2_w, lw.a2_b, r.tau, decay)
+      (qo, qn), (ko, kn), (vo, vn) = lw.cols["rq"], lw.cols["rk"], lw.cols["rv"]
+      K.linear_recurrence(P[:, qo:qo + qn], P[:, ko:ko + kn], P[:, vo:vo + vn], decay, None, d ** -0.5, st.S[j],
+                          inp.state_slots, inp.cu_q, o)
+    off, n = lw.mix_cols["rec"]
+    K.gated_rmsnorm(o, lw.rec_norm, P, lw.cols["rg"][0], self.c.rms_norm_eps, lw.spec.rec_scale, mix[:, off:off + n])
+
+  def _forward_mixed(self, x: torch.Tensor, inp: StepInputs) -> torch.Tensor:
+    """Layers of config.layer_specs on an fp32 residual stream h:
+      hn = h / rms(h) * g                       one scalar gain per norm (fused into the previous layer's residual add)
+      P  = hn @ in_w^T                          every projection of the layer in one GEMM, fp32 result
+      mix = [attn_scale * attention | rec_scale * recurrence]    both mixers read hn; outputs side by side along K
+      h += ls1 * (mix @ out_w^T) + ls2 * (gelu_tanh(gate) * up) @ down_w^T
+    Returns h (non-last shard) or logit_scale * head(norm(h rows inp.last_idx))."""
+    c, w = self.c, self.w
+    if c.has_state and (self.state is None or inp.state_slots is None):
+      raise RuntimeError("a model with recurrent layers needs a state pool and the step's state slots")
+    if self.shard.is_first_layer():
+      h = w.embed.index_select(0, x.view(-1).long())
+    else:
+      h = x.to(torch.float32).contiguous().clone()
+    T, D = h.shape
+    n = len(self.layer_ids)
+    last = self.shard.is_last_layer()
+    adt = (w.layers[self.layer_ids[0]].in_w if n else w.lm_head).dtype
+    bufs = {}
+
+    def rows(name: str, live: int, padded: int) -> torch.Tensor:
+      # activation rows whose K-padding columns stay zero: kernels only write the first `live` columns
+      key = (name, live, padded)
+      if key not in bufs:
+        bufs[key] = torch.zeros(T, padded, dtype=adt, device=h.device)
+      return bufs[key]
+    hn = rows("hn", D, -(-D // 128) * 128)
+    if n:
+      K.resid_scale_norm(h, gain=w.layers[self.layer_ids[0]].norm_g, eps=c.rms_norm_eps, out=hn)
+    for j, li in enumerate(self.layer_ids):
+      lw = w.layers[li]
+      s = lw.spec
+      P = self._proj(hn, lw.in_w)
+      live = sum(sz for _, sz in lw.mix_cols.values())
+      mix = rows("mix", live, lw.out_w.shape[1])
+      if s.attn is not None:
+        self._gated_attn(P, lw, j, inp, mix)
+      if s.rec is not None:
+        self._recurrence(P, lw, j, inp, mix)
+      y1 = self._proj(mix, lw.out_w)
+      y2 = None
+      if s.ff:
+        act = rows("act", s.ff, lw.down_w.shape[1])
+        K.gelu_mul(P, lw.cols["gate"][0], lw.cols["up"][0], s.ff, act)
+        y2 = self._proj(act, lw.down_w)
+      nxt = w.layers[self.layer_ids[j + 1]].norm_g if j + 1 < n else None
+      K.resid_scale_norm(h, y1, lw.ls1, y2, lw.ls2 if y2 is not None else None, gain=nxt, eps=c.rms_norm_eps,
+                         out=hn if nxt is not None else None)
+    if not last:
+      return h
+    hl = h.index_select(0, inp.last_idx)
+    xn = torch.zeros(hl.shape[0], hn.shape[1], dtype=adt, device=h.device)
+    K.resid_scale_norm(hl, gain=w.norm, eps=c.rms_norm_eps, out=xn)
+    logits = self._proj(xn, w.lm_head)[:, :c.vocab_size]
+    return logits * c.logit_scale
+
   # ------------------------------------------------------------------ forward
   @torch.inference_mode()
   def forward(self, x: torch.Tensor, inp: StepInputs) -> torch.Tensor:
     """x: token ids [T] (first shard) or hidden [T, D] bf16.  Returns hidden [T, D] (non-last shard)
     or fp32 logits [B, V] of each sequence's last token (last shard)."""
     c, w = self.c, self.w
+    if c.is_mixed:
+      return self._forward_mixed(x, inp)
     if self.shard.is_first_layer():
       h = K.embedding(x, w.embed)
       if inp.image_embeds is not None:  # LLaVA: projected image features replace the image-token rows

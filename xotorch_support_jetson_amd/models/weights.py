@@ -333,6 +333,14 @@ def prepare_for_decode(sw: "ShardWeights", keep_rowmajor: Iterable[str] = (), fp
     out.xot_layout = "stream_t" if transpose else "stream"
     return out
 
+  if sw.config.is_mixed:  # fused projections of mixed-layer models (bf16 runs; an fp32 run keeps vendor SGEMM layouts)
+    for lw in sw.layers.values():
+      if lw.in_w.dtype == torch.bfloat16:
+        lw.in_w, lw.out_w, lw.down_w = conv(lw.in_w), conv(lw.out_w), conv(lw.down_w)
+    if sw.lm_head is not None and sw.lm_head.dtype == torch.bfloat16:
+      sw.lm_head = conv(sw.lm_head)
+    return sw
+
   proj = conv8 if fp8 else conv
 
   def keep_logical(new, old):  # a converted weight keeps the padded tensor's logical shape
@@ -428,6 +436,9 @@ def random_weights(c: ModelConfig, shard: Shard, device: torch.device | str = "c
   """Deterministic per-layer random weights: layer i is identical whichever shard holds it, so a
   pipeline split reproduces the unsplit model exactly (the split-vs-full equivalence tests)."""
   dev = torch.device(device)
+  if c.is_mixed:
+    tensors = random_mixed_tensors(c, seed)
+    return mixed_weights(c, shard, tensors.__getitem__, dev, dtype)
   D, Fd, E = c.hidden_size, c.intermediate_size, c.num_experts
 
   def gen(tag: int):
@@ -554,6 +565,8 @@ def load_hf_weights(model_dir: str | Path, c: ModelConfig, shard: Shard, device=
   """Read only this shard's tensors (mmap'd safetensors, one tensor at a time) into the fused layout."""
   from safetensors import safe_open
   model_dir = Path(model_dir)
+  if c.is_mixed:
+    return load_mixed_weights(model_dir, c, shard, device, dtype)
   raw = _weight_map(model_dir)
   wm = {canonical_name(k): (k, f) for k, f in raw.items()}
   handles = {}
@@ -647,3 +660,191 @@ def from_hf_state_dict(sd: Dict[str, torch.Tensor], c: ModelConfig, shard: Shard
   with tempfile.TemporaryDirectory() as d:
     save_file({k: v.contiguous() for k, v in sd.items()}, os.path.join(d, "model.safetensors"))
     return load_hf_weights(d, c, shard, device, dtype)
+
+
+# -------------------------------------------------------------------- layers of differing mixers (Tarepel)
+def _up(n: int, m: int) -> int:
+  return -(-n // m) * m
+
+
+@dataclass
+class MixedLayerWeights:
+  """One layer of a mixed-layer model (config.MixedLayerSpec) in the device layout.
+
+  Every projection that reads the layer's one normed input is a row block of `in_w` [Np, Dp] (one GEMM per layer):
+  `cols[name] = (offset, size)` addresses its slice of the fp32 result.  The mixers' outputs are concatenated along
+  K into one row buffer for `out_w` [Dn, Kp] = [attention o | recurrence o]; `down_w` [Dn, Fp] is the feed-forward's
+  down projection.  Rows / columns are zero-padded to the GEMM tiles (Np, Dn: 64; Dp, Kp, Fp: 128).  Projection
+  weights have the compute dtype (bf16, or fp32 for an all-fp32 run); everything a norm, a score or a recurrence
+  reads is fp32."""
+  spec: object
+  in_w: torch.Tensor
+  cols: Dict[str, tuple]
+  out_w: torch.Tensor
+  mix_cols: Dict[str, tuple]  # "attn" / "rec": (offset, size) in the mixers' output row
+  norm_g: torch.Tensor  # [1] fp32
+  ls1: torch.Tensor  # [D] fp32
+  ls2: Optional[torch.Tensor] = None
+  down_w: Optional[torch.Tensor] = None
+  attn_pb: Optional[torch.Tensor] = None  # [H] fp32
+  conv_w: Optional[torch.Tensor] = None  # [2 G d + H dv, taps] fp32 (q | k | v channels)
+  A_log: Optional[torch.Tensor] = None
+  dt_bias: Optional[torch.Tensor] = None
+  rec_norm: Optional[torch.Tensor] = None  # [dv] fp32
+  a2_w: Optional[torch.Tensor] = None  # [H d, rank] fp32
+  a2_b: Optional[torch.Tensor] = None
+  router: Optional[torch.Tensor] = None  # (dense feed-forward only; kept for code that asks)
+
+  def tensors(self) -> Dict[str, torch.Tensor]:
+    return {k: v for k, v in self.__dict__.items() if isinstance(v, torch.Tensor)}
+
+
+def mixed_layer_names(spec, p: str) -> Dict[str, list]:
+  """Checkpoint tensor names of one layer: {"in": [(column name, tensor)], "out": [(mix name, tensor)], ...}."""
+  if spec.kind == "parallel":
+    a, r = p + "mix.left.", p + "mix.right."
+    return {"in": [("aq", a + "q"), ("ak", a + "k"), ("rq", r + "q"), ("rk", r + "k"), ("rv", r + "v"), ("rg", r + "g"),
+                   ("rb", r + "b"), ("ra", r + "a")],
+            "out": [("attn", a + "o"), ("rec", r + "o")], "pb": a + "pb", "conv": [r + "q.conv", r + "k.conv", r + "v.conv"],
+            "A_log": r + "A_log", "dt_bias": r + "dt_bias", "rec_norm": r + "norm"}
+  m = p + "mix."
+  return {"in": [("rq", m + "q"), ("rk", m + "k"), ("rv", m + "v"), ("rg", m + "g"), ("ra1", m + "a1")],
+          "out": [("rec", m + "o")], "rec_norm": m + "norm", "a2": m + "a2", "a2_b": m + "a2.b"}
+
+
+def build_mixed_layer(spec, get, p: str, D: int, device, dtype) -> MixedLayerWeights:
+  """Assemble one layer from `get(name) -> fp32 CPU tensor` (a checkpoint reader or a random generator)."""
+  names = mixed_layer_names(spec, p)
+  blocks = [(n, get(t)) for n, t in names["in"]]
+  if spec.ff:
+    blocks += [("gate", get(p + "mlp.gate")), ("up", get(p + "mlp.up"))]
+  cols, off = {}, 0
+  for n, w in blocks:
+    cols[n] = (off, w.shape[0])
+    off += w.shape[0]
+  Dp = _up(D, 128)
+  in_w = torch.zeros(_up(off, 64), Dp)
+  in_w[:off, :D] = torch.cat([w for _, w in blocks], 0)
+  outs = [(n, get(t)) for n, t in names["out"]]
+  mix_cols, k = {}, 0
+  for n, w in outs:
+    mix_cols[n] = (k, w.shape[1])
+    k += w.shape[1]
+  out_w = torch.zeros(_up(D, 64), _up(k, 128))
+  out_w[:D, :k] = torch.cat([w for _, w in outs], 1)
+
+  def dev(t, dt=torch.float32):
+    return t.to(device=device, dtype=dt).contiguous()
+  lw = MixedLayerWeights(spec, dev(in_w, dtype), cols, dev(out_w, dtype), mix_cols, dev(get(p + "norm1").reshape(1)),
+                         dev(get(p + "ls1")))
+  if spec.ff:
+    down = get(p + "mlp.down")
+    dw = torch.zeros(_up(D, 64), _up(spec.ff, 128))
+    dw[:D, :spec.ff] = down
+    lw.down_w, lw.ls2 = dev(dw, dtype), dev(get(p + "ls2"))
+  if "pb" in names:
+    lw.attn_pb = dev(get(names["pb"]))
+  if "conv" in names:
+    lw.conv_w = dev(torch.cat([get(n) for n in names["conv"]], 0))
+    lw.A_log, lw.dt_bias = dev(get(names["A_log"])), dev(get(names["dt_bias"]))
+  if "a2" in names:
+    lw.a2_w, lw.a2_b = dev(get(names["a2"])), dev(get(names["a2_b"]))
+  lw.rec_norm = dev(get(names["rec_norm"]))
+  return lw
+
+
+def mixed_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
+  """Name -> shape of every tensor of a mixed-layer checkpoint (random init, checkpoint validation)."""
+  D, out = c.hidden_size, {}
+  out["embed"] = (c.vocab_size, D)
+  for i, s in enumerate(c.layer_specs):
+    p = f"l{i}."
+    out[p + "norm1"], out[p + "ls1"] = (), (D,)
+    if s.attn is not None:
+      a, m = s.attn, p + "mix.left."
+      out[m + "q"], out[m + "k"], out[m + "pb"], out[m + "o"] = (a.heads * a.dim, D), (a.kv_heads * a.dim, D), (a.heads,), \
+        (D, a.heads * a.vdim)
+    r = s.rec
+    if r is not None and r.rule == "delta":
+      m = p + "mix.right."
+      for n, rows in (("q", r.kv_heads * r.dim), ("k", r.kv_heads * r.dim), ("v", r.heads * r.vdim)):
+        out[m + n], out[m + n + ".conv"] = (rows, D), (rows, r.conv)
+      out[m + "b"], out[m + "a"], out[m + "A_log"], out[m + "dt_bias"] = (r.heads, D), (r.heads, D), (r.heads,), (r.heads,)
+      out[m + "norm"], out[m + "g"], out[m + "o"] = (r.vdim,), (r.heads * r.vdim, D), (D, r.heads * r.vdim)
+    elif r is not None:
+      m, rank = p + "mix.", r.rank or 16
+      out[m + "q"], out[m + "k"], out[m + "v"] = (r.heads * r.dim, D), (r.heads * r.dim, D), (r.heads * r.vdim, D)
+      out[m + "g"], out[m + "o"], out[m + "norm"] = (r.heads * r.vdim, D), (D, r.heads * r.vdim), (r.vdim,)
+      out[m + "a1"], out[m + "a2"], out[m + "a2.b"] = (rank, D), (r.heads * r.dim, rank), (r.heads * r.dim,)
+    if s.ff:
+      out[p + "mlp.gate"], out[p + "mlp.up"], out[p + "mlp.down"], out[p + "ls2"] = (s.ff, D), (s.ff, D), (D, s.ff), (D,)
+  out["final.norm"], out["head"] = (), (c.vocab_size, D)
+  return out
+
+
+def random_mixed_tensors(c: ModelConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
+  """Deterministic random checkpoint of a mixed-layer architecture, values rounded to bf16 (as a stored checkpoint's
+  are): projections ~ N(0, 1/sqrt(fan_in)), gains / layer scales / biases of order one so every mechanism shows."""
+  out = {}
+  for j, (name, shape) in enumerate(mixed_tensor_shapes(c).items()):
+    g = torch.Generator().manual_seed(seed * 1_000_003 + 7919 * j + 17)
+    leaf = name.split(".")[-1]
+    if name.endswith(".conv"):
+      t = torch.randn(shape, generator=g) * 0.5
+    elif leaf in ("norm1",) or name == "final.norm":
+      t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+    elif leaf in ("ls1", "ls2"):
+      t = 0.5 + 0.1 * torch.randn(shape, generator=g)
+    elif leaf == "norm":
+      t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+    elif leaf in ("pb", "dt_bias"):
+      t = torch.randn(shape, generator=g) - (2.0 if leaf == "pb" else 0.0)
+    elif leaf == "A_log":
+      t = torch.rand(shape, generator=g) * 1.5 - 2.0
+    elif leaf == "b" and len(shape) == 1:  # a2.b: decays close to one
+      t = 3.0 + torch.randn(shape, generator=g)
+    elif name == "embed":
+      t = torch.randn(shape, generator=g)
+    else:
+      t = torch.randn(shape, generator=g) / shape[-1] ** 0.5
+    out[name] = t.to(torch.bfloat16).float()
+  return out
+
+
+def mixed_weights(c: ModelConfig, shard: Shard, get, device, dtype) -> ShardWeights:
+  """ShardWeights of a mixed-layer model from `get(name) -> fp32 CPU tensor`."""
+  sw = ShardWeights(c, shard)
+  D = c.hidden_size
+  for i in shard.layers():
+    sw.layers[i] = build_mixed_layer(c.layer_specs[i], get, f"l{i}.", D, device, dtype)
+  if shard.is_first_layer():
+    sw.embed = get("embed").to(device=device, dtype=torch.float32).contiguous()  # gathered into the fp32 residual
+  if shard.is_last_layer():
+    sw.norm = get("final.norm").reshape(1).to(device=device, dtype=torch.float32)
+    head = torch.zeros(_up(c.vocab_size, 64), _up(D, 128))
+    head[:c.vocab_size, :D] = get("head")
+    sw.lm_head = head.to(device=device, dtype=dtype).contiguous()
+  return sw
+
+
+def load_mixed_weights(model_dir: Path, c: ModelConfig, shard: Shard, device, dtype) -> ShardWeights:
+  """Tarepel checkpoint (flat names: embed, l<i>.norm1, l<i>.mix.*, l<i>.mlp.*, l<i>.ls1 / ls2, final.norm, head).
+  The decay rank of a gated-linear-attention layer is the a1 tensor's row count."""
+  from safetensors import safe_open
+  wm = _weight_map(Path(model_dir))
+  handles = {}
+
+  def get(name: str) -> torch.Tensor:
+    if name not in wm:
+      raise KeyError(f"checkpoint has no tensor {name!r}")
+    f = wm[name]
+    if f not in handles:
+      handles[f] = safe_open(str(Path(model_dir) / f), framework="pt")
+    return handles[f].get_tensor(name).float()
+  want = mixed_tensor_shapes(c)
+  for name, shape in want.items():
+    if name.split(".")[0] in ("embed", "final", "head") or int(name.split(".")[0][1:]) in shard.layers():
+      got = tuple(get(name).shape) if not name.endswith((".a1", ".a2")) else None
+      if got is not None and got != tuple(shape):
+        raise ValueError(f"{name}: checkpoint shape {got}, config says {tuple(shape)}")
+  return mixed_weights(c, shard, get, device, dtype)

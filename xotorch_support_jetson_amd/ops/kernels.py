@@ -435,3 +435,61 @@ def moe_route_ds(logits, bias, k: int, n_group: int, topk_group: int, method: in
   require().moe_route_ds(logits.contiguous(), bias, int(k), int(n_group), int(topk_group), int(method), bool(sigmoid),
                          bool(norm), float(scale), _route_counters(dev), *outs)
   return outs
+
+
+# ------------------------------------------------------------------ mixers on an fp32 residual stream (csrc/mixers.hip)
+# P is a fused projection's fp32 output [T, n]; *_off are column offsets into it.  Outputs are preallocated by the
+# caller (graph-capturable); activation outputs may be column slices of a wider row buffer.
+def _mix(name: str, on_gpu: bool):
+  return getattr(require(), name) if on_gpu else getattr(ref, name)
+
+
+def resid_scale_norm(x, y1=None, s1=None, y2=None, s2=None, gain=None, eps: float = 1e-5, out=None) -> None:
+  """fp32 residual rows x [T, D] += s1 * y1 (+ s2 * y2) in place (per-channel scales; y rows may be wider than
+  D), then, with `out`, out[:, :D] = x / sqrt(mean(x^2) + eps) * gain (gain: one fp32 number on the device)."""
+  _mix("resid_scale_norm", _gpu(x))(x, y1, s1, y2, s2, gain, float(eps), out)
+
+
+def gelu_mul(P, gate_off: int, up_off: int, F: int, out) -> None:
+  """out[:, :F] = gelu_tanh(P[:, gate_off : +F]) * P[:, up_off : +F]  (out rows may be wider: K padding)."""
+  _mix("gelu_mul", _gpu(P))(P, int(gate_off), int(up_off), int(F), out)
+
+
+def rope_kv_store(P, q_off: int, k_off: int, v_off: int, H: int, G: int, d: int, R: int, pos, cos_sin, slots, q_out,
+                  k_cache, v_cache) -> None:
+  """Rotate-half RoPE on the first R dims of every q / k head (pairs (i, i + R/2)); q -> q_out [T, H, d], the
+  rotated key and the value (v_off < 0: the key before rotation) -> paged caches [pages, G, 64, d] at `slots`."""
+  _mix("rope_kv_store", _gpu(P))(P, int(q_off), int(k_off), int(v_off), int(H), int(G), int(d), int(R), pos, cos_sin,
+                                 slots, q_out, k_cache, v_cache)
+
+
+def attn_gated_chunk(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, scale: float, chunk: int, out_scale: float,
+                     out) -> None:
+  """out [T, H d] = out_scale * sum over the keys j <= i of query i's chunk (floor(i / chunk) == floor(j / chunk))
+  of sigmoid(q_i . k_j * scale + pb[head]) v_j; positions count from each sequence's start."""
+  _mix("attn_gated_chunk", _gpu(q))(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, float(scale), int(chunk),
+                                    float(out_scale), out)
+
+
+def delta_prep(P, x_off: int, b_off: int, a_off: int, conv_w, conv_state, state_slots, cu_q, A_log, dt_bias, H: int,
+               G: int, d: int, dv: int, qkv, beta, decay) -> None:
+  """Delta-rule inputs of a step and the convolution state's update (see csrc/mixers.hip delta_prep)."""
+  _mix("delta_prep", _gpu(P))(P, int(x_off), int(b_off), int(a_off), conv_w, conv_state, state_slots, cu_q, A_log, dt_bias,
+                              int(H), int(G), int(d), int(dv), qkv, beta, decay)
+
+
+def gla_prep(P, a1_off: int, a2, a2_b, tau: float, decay) -> None:
+  """decay [T, H d] = sigmoid(z)^(1/tau), z = a2 P[:, a1_off : +rank] + a2_b."""
+  _mix("gla_prep", _gpu(P))(P, int(a1_off), a2, a2_b, float(tau), decay)
+
+
+def linear_recurrence(q, k, v, decay, beta, q_scale: float, state, state_slots, cu_q, out) -> None:
+  """Per sequence and value head, token by token on the fp32 state [slots, H, d, dv] (updated in place):
+  beta given (delta rule, decay [T, H]):  S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q
+  else (decay [T, H d] per key channel):  S = diag(a) S + k v^T; o = S^T q.      q is scaled by q_scale."""
+  _mix("linear_recurrence", _gpu(q))(q, k, v, decay, beta, float(q_scale), state, state_slots, cu_q, out)
+
+
+def gated_rmsnorm(o, w, P, g_off: int, eps: float, out_scale: float, out) -> None:
+  """out [T, H dv] = o / rms(o per head) * w * silu(P[:, g_off : +H dv]) * out_scale."""
+  _mix("gated_rmsnorm", _gpu(o))(o, w, P, int(g_off), float(eps), float(out_scale), out)

@@ -229,3 +229,120 @@ def moe_route_ds(logits, bias, k: int, n_group: int, topk_group: int, method: in
   if norm:
     topw = topw / (topw.sum(-1, keepdim=True) + 1e-20)
   return topw * scale, topi
+
+
+# ------------------------------------------------------------------ mixers on an fp32 residual stream
+# Torch twins of csrc/mixers.hip.  P is a fused projection's output [T, n] (fp32 on a GPU; whatever the CPU GEMM
+# returned here), addressed by column offsets.  Per-sequence loops are fine: this is the CPU path.
+def resid_scale_norm(x, y1, s1, y2, s2, gain, eps, out):
+  """x += s1 * y1 (+ s2 * y2) in place; out = x / sqrt(mean(x^2) + eps) * gain."""
+  D = x.shape[1]
+  if y1 is not None:
+    a = s1.float() * y1[:, :D].float()
+    if y2 is not None:
+      a = a + s2.float() * y2[:, :D].float()
+    x += a
+  if out is not None:
+    out[:, :D] = (x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * gain.float()).to(out.dtype)
+
+
+def gelu_mul(P, gate_off, up_off, Fd, out):
+  z, u = P[:, gate_off:gate_off + Fd].float(), P[:, up_off:up_off + Fd].float()
+  out[:, :Fd] = (0.5 * z * (1 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3))) * u).to(out.dtype)
+
+
+def rope_kv_store(P, q_off, k_off, v_off, H, G, d, R, pos, cos_sin, slots, q_out, k_cache, v_cache):
+  T = P.shape[0]
+  q = P[:, q_off:q_off + H * d].float().reshape(T, H, d)
+  k = P[:, k_off:k_off + G * d].float().reshape(T, G, d)
+  v = k if v_off < 0 else P[:, v_off:v_off + G * d].float().reshape(T, G, d)
+  half = R // 2
+
+  def rot(x):
+    if R == 0:
+      return x
+    cs = cos_sin[pos.long()]
+    c, s = cs[:, None, :half], cs[:, None, half:]
+    a, b = x[..., :half], x[..., half:R]
+    return torch.cat([a * c - b * s, b * c + a * s, x[..., R:]], -1)
+  q_out.copy_(rot(q).to(q_out.dtype))
+  ok = slots >= 0
+  s = slots[ok].long()
+  k_cache[s // PAGE, :, s % PAGE] = rot(k)[ok].to(k_cache.dtype)
+  v_cache[s // PAGE, :, s % PAGE] = v[ok].to(v_cache.dtype)
+
+
+def attn_gated_chunk(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, scale, chunk, out_scale, out):
+  T, H, d = q.shape
+  G = k_cache.shape[1]
+  for b in range(ctx_lens.numel()):
+    t0, t1, n = int(cu_q[b]), int(cu_q[b + 1]), int(ctx_lens[b])
+    if n <= 0 or t1 == t0:
+      continue
+    npg = -(-n // PAGE)
+    pages = block_tables[b, :npg].long()
+    k = k_cache[pages].permute(0, 2, 1, 3).reshape(npg * PAGE, G, d)[:n].float().repeat_interleave(H // G, 1)
+    v = v_cache[pages].permute(0, 2, 1, 3).reshape(npg * PAGE, G, d)[:n].float().repeat_interleave(H // G, 1)
+    qpos = torch.arange(n - (t1 - t0), n)[:, None]
+    kpos = torch.arange(n)[None, :]
+    vis = (kpos <= qpos) & (kpos // chunk == qpos // chunk)
+    s = torch.einsum("shd,thd->hst", q[t0:t1].float(), k) * scale + pb.float()[:, None, None]
+    w = torch.sigmoid(s) * vis
+    o = torch.einsum("hst,thd->shd", w, v) * out_scale
+    out[t0:t1] = o.reshape(t1 - t0, H * d).to(out.dtype)
+
+
+def delta_prep(P, x_off, b_off, a_off, conv_w, conv_state, state_slots, cu_q, A_log, dt_bias, H, G, d, dv, qkv, beta, decay):
+  C = 2 * G * d + H * dv
+  taps = conv_w.shape[1]
+  for b in range(state_slots.numel()):
+    t0, t1, slot = int(cu_q[b]), int(cu_q[b + 1]), int(state_slots[b])
+    if slot < 0 or t1 == t0:
+      continue
+    x = torch.cat([conv_state[slot], P[t0:t1, x_off:x_off + C].float()], 0)  # [taps - 1 + n, C]
+    y = sum(conv_w[:, j].float() * x[j:j + t1 - t0] for j in range(taps))
+    y = F.silu(y)
+    qk = y[:, :2 * G * d].reshape(t1 - t0, 2 * G, d)
+    qk = qk / torch.sqrt(qk.pow(2).sum(-1, keepdim=True) + 1e-6)
+    qk[:, :G] *= d ** -0.5
+    qkv[t0:t1] = torch.cat([qk.reshape(t1 - t0, -1), y[:, 2 * G * d:]], 1)
+    conv_state[slot] = x[x.shape[0] - (taps - 1):]
+    beta[t0:t1] = torch.sigmoid(P[t0:t1, b_off:b_off + H].float())
+    decay[t0:t1] = torch.exp(-torch.exp(A_log.float()) * F.softplus(P[t0:t1, a_off:a_off + H].float() + dt_bias.float()))
+
+
+def gla_prep(P, a1_off, a2, a2_b, tau, decay):
+  z = P[:, a1_off:a1_off + a2.shape[1]].float() @ a2.float().t() + a2_b.float()
+  decay.copy_(torch.exp(F.logsigmoid(z) / tau))
+
+
+def linear_recurrence(q, k, v, decay, beta, q_scale, state, state_slots, cu_q, out):
+  _, H, d, dv = state.shape
+  G = q.shape[1] // d
+  rep = H // G
+  for b in range(state_slots.numel()):
+    t0, t1, slot = int(cu_q[b]), int(cu_q[b + 1]), int(state_slots[b])
+    if slot < 0 or t1 == t0:
+      continue
+    S = state[slot]
+    for t in range(t0, t1):
+      qt = (q[t].float() * q_scale).reshape(G, d).repeat_interleave(rep, 0)
+      kt = k[t].float().reshape(G, d).repeat_interleave(rep, 0)
+      vt = v[t].float().reshape(H, dv)
+      if beta is not None:
+        S *= decay[t].reshape(H, 1, 1)
+        u = beta[t].reshape(H, 1) * (vt - torch.einsum("hdv,hd->hv", S, kt))
+        S += kt[:, :, None] * u[:, None, :]
+      else:
+        S *= decay[t].reshape(H, d, 1)
+        S += kt[:, :, None] * vt[:, None, :]
+      out[t] = torch.einsum("hdv,hd->hv", S, qt).reshape(-1)
+
+
+def gated_rmsnorm(o, w, P, g_off, eps, out_scale, out):
+  T = P.shape[0]
+  dv = w.numel()
+  x = o.reshape(T, -1, dv).float()
+  gate = P[:, g_off:g_off + x.shape[1] * dv].float().reshape(T, -1, dv)
+  y = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float() * F.silu(gate) * out_scale
+  out.copy_(y.reshape(T, -1).to(out.dtype))

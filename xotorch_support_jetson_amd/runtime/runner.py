@@ -15,7 +15,7 @@ import torch
 
 from ..inference.shard import Shard
 from ..models.config import ModelConfig
-from ..models.transformer import KVCache, ShardModel, StepInputs
+from ..models.transformer import KVCache, ShardModel, StatePool, StepInputs
 from ..models.weights import ShardWeights, prepare_for_decode, random_weights
 from ..ops import linear as linear_mod
 
@@ -31,6 +31,38 @@ def _block_manager(num_pages: int):
     return BlockManager(num_pages, PAGE)
 
 
+class SlotManager:
+  """State slots of models with recurrent layers: one slot per live request, handed out on admission and returned
+  when the request ends (lowest free slot first, so a small pool is reused at once)."""
+
+  def __init__(self, slots: int):
+    self.slots = slots
+    self._free: List[int] = list(range(slots - 1, -1, -1))
+    self._of: Dict[str, int] = {}
+
+  @property
+  def num_free(self) -> int:
+    return len(self._free)
+
+  def has(self, rid: str) -> bool:
+    return rid in self._of
+
+  def slot(self, rid: str) -> int:
+    return self._of[rid]
+
+  def acquire(self, rid: str) -> int:
+    if not self._free:
+      raise RuntimeError(f"state slots exhausted: all {self.slots} are held by live requests")
+    s = self._of[rid] = self._free.pop()
+    return s
+
+  def release(self, rid: str) -> None:
+    s = self._of.pop(rid, None)
+    if s is not None:
+      self._free.append(s)
+      self._free.sort(reverse=True)
+
+
 def _bucket(n: int) -> int:
   for b in (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 160, 192, 256, 320, 384, 448, 512):
     if n <= b:
@@ -41,14 +73,21 @@ def _bucket(n: int) -> int:
 class ShardRunner:
   def __init__(self, config: ModelConfig, shard: Shard, device: torch.device | str = "cpu",
                weights: Optional[ShardWeights] = None, num_pages: Optional[int] = None, max_batch: int = 128,
-               max_ctx: int = 4096, kv_mem_fraction: float = 0.85, seed: int = 0, use_graphs: Optional[bool] = None):
+               max_ctx: int = 4096, kv_mem_fraction: float = 0.85, seed: int = 0, use_graphs: Optional[bool] = None,
+               dtype: torch.dtype = torch.bfloat16):
+    """dtype: the compute dtype of mixed-layer models (bfloat16, or float32 for an all-fp32 run: fp32 weights, caches
+    and vendor SGEMMs); the other architectures serve in bfloat16 only."""
     self.config = config
+    self.dtype = dtype
+    if dtype != torch.bfloat16 and not config.is_mixed:
+      raise ValueError(f"{config.model_type} serves in bfloat16 only")
     self.shard = shard
     self.device = torch.device(device)
     if self.device.type == "cuda":
       torch.cuda.set_device(self.device)
     self._random_weights, self._seed = weights is None, seed
-    self.weights = weights if weights is not None else random_weights(config, shard, self.device, seed=seed)
+    self.weights = weights if weights is not None else random_weights(config, shard, self.device, seed=seed,
+                                                                      **({"dtype": dtype} if config.is_mixed else {}))
     if self.device.type == "cuda" and os.environ.get("XOT_SHUFFLE", "1") == "1":
       # projection weights -> pre-shuffled MFMA-fragment layout: gemm_stream for decode-shaped M, gemm_big
       # (256 x 256 LDS-DMA tiles, fused SiLU / residual epilogues) for large decode batches and prefill
@@ -61,7 +100,8 @@ class ShardRunner:
       self.weight_dtype = os.environ.get("XOT_WEIGHT_DTYPE", "bf16")
       prepare_for_decode(self.weights, keep_rowmajor=keep, fp8=self.weight_dtype == "fp8")
     n_layers = shard.get_layer_count()
-    per_page = KVCache.bytes_per_page(config, n_layers)
+    per_page = KVCache.bytes_per_page(config, n_layers, shard.layers(), torch.empty(0, dtype=dtype).element_size()) \
+      if config.is_mixed else KVCache.bytes_per_page(config, n_layers)
     if num_pages is None:
       if self.device.type == "cuda":
         free, _ = torch.cuda.mem_get_info(self.device)
@@ -70,12 +110,17 @@ class ShardRunner:
       else:
         num_pages = max(64, (max_batch * max_ctx) // PAGE // 4)
       num_pages = min(num_pages, max_batch * (-(-max_ctx // PAGE)) + 16)
-    self.kv = KVCache(config, n_layers, num_pages, self.device)
+    self.kv = KVCache(config, n_layers, num_pages, self.device, dtype, shard.layers()) if config.is_mixed else \
+      KVCache(config, n_layers, num_pages, self.device)
     self.bm = _block_manager(num_pages)
+    # recurrent layers: one state slot per live request (max_batch of them), cleared on admission
+    self.sm = SlotManager(max_batch) if config.has_state else None
+    self.state = StatePool(config, shard.layers(), max_batch, self.device) if config.has_state else None
     self.max_ctx = max_ctx
     self.max_batch = max_batch
     self.width = -(-max_ctx // PAGE)
     self.model = ShardModel(self.weights, self.kv, max_batch=max_batch, max_ctx=max_ctx)
+    self.model.state = self.state
     if use_graphs is None:
       # MoE routing runs on the device too (moe_route + grouped GEMMs), so every model is capturable
       use_graphs = self.device.type == "cuda" and os.environ.get("XOT_GRAPHS", "1") == "1"
@@ -97,7 +142,8 @@ class ShardRunner:
       st = {"tables": torch.zeros(max_batch, self.width, dtype=torch.int32),
             "ctx": torch.zeros(max_batch, dtype=torch.int32),
             "pos": torch.zeros(bmax, dtype=torch.int32),  # decode-step positions / slots (graph inputs)
-            "slots": torch.zeros(bmax, dtype=torch.int64)}
+            "slots": torch.zeros(bmax, dtype=torch.int64),
+            "sslots": torch.zeros(bmax, dtype=torch.int32)}  # state slots (recurrent layers)
       if self.device.type == "cuda":
         # pinned: an async copy out of pageable memory may wait for the stream to drain, i.e. for the step
         # already running, which would forbid queueing the next decode step behind it
@@ -112,6 +158,7 @@ class ShardRunner:
     st = self._sets[i]
     self._set_idx = i
     self._tables_host, self._ctx_host, self._pos_host, self._slots_host = st["tables"], st["ctx"], st["pos"], st["slots"]
+    self._sslots_host = st["sslots"]
     self._tables_cls = st["cls"]
 
   def _reuse_staging(self) -> None:
@@ -129,6 +176,11 @@ class ShardRunner:
       ev.record()
       self._sets[self._set_idx]["event"] = ev
 
+  @property
+  def hidden_dtype(self) -> torch.dtype:
+    """dtype of the hidden states that travel between shards (mixed-layer models carry an fp32 residual stream)."""
+    return torch.float32 if self.config.is_mixed else torch.bfloat16
+
   # ------------------------------------------------------------------ bookkeeping
   def has(self, rid: str) -> bool:
     return self.bm.has(rid)
@@ -138,21 +190,38 @@ class ShardRunner:
 
   def free(self, rid: str) -> None:
     self.bm.free(rid)
+    if self.sm is not None:
+      self.sm.release(rid)
 
   def can_admit(self, rid: str, n_new: int) -> bool:
+    if self.sm is not None and not self.sm.has(rid) and self.sm.num_free == 0:
+      return False
     return self.bm.can_append(rid, n_new) and self.num_tokens(rid) + n_new <= self.max_ctx
 
+  def _state_slot(self, rid: str) -> int:
+    """The request's state slot; a request seen for the first time gets a cleared one."""
+    if self.sm.has(rid):
+      return self.sm.slot(rid)
+    if self.bm.has(rid) and self.bm.num_tokens(rid) > 0:
+      raise RuntimeError(f"request {rid} holds cached tokens but no recurrent state")
+    s = self.sm.acquire(rid)
+    self.state.clear(s)
+    return s
+
   def truncate(self, rid: str, n: int) -> None:
+    if self.sm is not None and n != self.num_tokens(rid):
+      raise RuntimeError("a recurrent state cannot be rolled back to an earlier token")
     self.bm.truncate(rid, n)
 
   # ------------------------------------------------------------------ step inputs
-  def _prepare(self, rids: Sequence[str], qlens: Sequence[int]) -> StepInputs:
+  def _prepare(self, rids: Sequence[str], qlens: Sequence[int], logit_rows: Optional[Sequence[int]] = None) -> StepInputs:
     if len(rids) > self.max_batch:
       raise ValueError(f"batch {len(rids)} exceeds max_batch {self.max_batch}")
     self._reuse_staging()
     pos: List[int] = []
     slots: List[int] = []
     cu = [0]
+    sslots = [self._state_slot(rid) for rid in rids] if self.sm is not None else None
     for rid, n in zip(rids, qlens):
       start = self.num_tokens(rid)
       if start + n > self.max_ctx:
@@ -160,6 +229,8 @@ class ShardRunner:
       slots += self.bm.append(rid, n)
       pos += self.model.rope_pos(start, n)
       cu.append(cu[-1] + n)
+    if logit_rows is not None and any(not 0 <= r < cu[-1] for r in logit_rows):
+      raise ValueError("logit_rows must index the step's tokens")
     B = len(rids)
     self.bm.fill_batch(list(rids), self._tables_host[:B].numpy(), self._ctx_host[:B].numpy())
     dev = self.device
@@ -170,24 +241,29 @@ class ShardRunner:
       block_tables=self._tables_host[:B].to(dev, non_blocking=non_blocking),
       ctx_lens=self._ctx_host[:B].to(dev, non_blocking=non_blocking),
       cu_q=torch.tensor(cu, dtype=torch.int32).to(dev, non_blocking=nb),
-      last_idx=torch.tensor([c - 1 for c in cu[1:]], dtype=torch.int64).to(dev, non_blocking=nb),
+      last_idx=torch.tensor([c - 1 for c in cu[1:]] if logit_rows is None else list(logit_rows),
+                            dtype=torch.int64).to(dev, non_blocking=nb),
       max_qlen=max(qlens),
       decode=all(q == 1 for q in qlens),
+      state_slots=None if sslots is None else torch.tensor(sslots, dtype=torch.int32).to(dev, non_blocking=nb),
     )
     self._mark_staged()
     return inp
 
   # ------------------------------------------------------------------ forward
   def forward(self, rids: Sequence[str], qlens: Sequence[int], x: torch.Tensor,
-              image_embeds: Optional[torch.Tensor] = None) -> torch.Tensor:
+              image_embeds: Optional[torch.Tensor] = None, logit_rows: Optional[Sequence[int]] = None) -> torch.Tensor:
     """Run this shard for the given requests.  x = token ids [sum(qlens)] (first shard) or hidden
     [sum(qlens), D].  Allocates KV slots for the new tokens.  Returns hidden [T, D] or, on the last
     shard, fp32 logits [len(rids), V] of each request's last token.  image_embeds (LLaVA, first shard):
-    projected image features for the image-token rows of x, in order."""
+    projected image features for the image-token rows of x, in order.
+    logit_rows (last shard): rows of x whose logits to return instead of each request's last token's, [len(logit_rows), V]
+    (replaying recorded traffic, scoring a prompt)."""
     x = x.to(self.device, non_blocking=True)
-    if self.use_graphs and image_embeds is None and all(q == 1 for q in qlens) and len(rids) <= self.max_batch:
+    if (self.use_graphs and image_embeds is None and logit_rows is None and all(q == 1 for q in qlens)
+        and len(rids) <= self.max_batch):
       return self._decode_graph(rids, x)
-    inp = self._prepare(rids, qlens)
+    inp = self._prepare(rids, qlens, logit_rows)
     if image_embeds is not None:
       inp.image_embeds = image_embeds.to(self.device)
     return self.model.forward(x, inp)
@@ -219,6 +295,7 @@ class ShardRunner:
     self._reuse_staging()
     pos, slots = [], []
     most = 0
+    sslots = [self._state_slot(rid) for rid in rids] if self.sm is not None else None
     for rid in rids:
       start = self.num_tokens(rid)
       if start + 1 > self.max_ctx:
@@ -238,6 +315,9 @@ class ShardRunner:
     self._slots_host[:Bp] = torch.tensor(slots + [-1] * pad, dtype=torch.int64)
     g["pos"].copy_(self._pos_host[:Bp], non_blocking=True)
     g["slots"].copy_(self._slots_host[:Bp], non_blocking=True)
+    if sslots is not None:
+      self._sslots_host[:Bp] = torch.tensor(sslots + [-1] * pad, dtype=torch.int32)
+      g["sslots"].copy_(self._sslots_host[:Bp], non_blocking=True)
     self._ctx_host[B:Bp] = 0
     g["tables"].copy_(tables[:Bp], non_blocking=True)
     g["ctx"].copy_(self._ctx_host[:Bp], non_blocking=True)
@@ -292,8 +372,12 @@ class ShardRunner:
     if self.shard.is_first_layer():
       g["x"] = torch.zeros(Bp, dtype=torch.int32, device=dev)
     else:
-      g["x"] = torch.zeros(Bp, c.hidden_size, dtype=torch.bfloat16, device=dev)
+      g["x"] = torch.zeros(Bp, c.hidden_size, dtype=self.hidden_dtype, device=dev)
     inp = StepInputs(g["pos"], g["slots"], g["tables"], g["ctx"], g["cu"], g["last"], 1, True)
+    if self.sm is not None:
+      # warm-up and capture run on padding rows only (state slot -1, no KV slot): no request's state is touched
+      g["sslots"] = torch.full((Bp,), -1, dtype=torch.int32, device=dev)
+      inp.state_slots = g["sslots"]
     # warm up eagerly (also settles the GEMM policy for these shapes) on a side stream
     s = torch.cuda.Stream(dev)
     s.wait_stream(torch.cuda.current_stream(dev))
