@@ -510,8 +510,16 @@ class ShardedInferenceEngine(InferenceEngine):
     tokens and prefill prompts mix; a prompt longer than the budget runs alone, chunked)."""
     cap = self.runner.max_batch if self.runner is not None else 1
     batch, rest, tokens = [], [], 0
+    sm = getattr(self.runner, "sm", None)  # models with recurrent layers: a new request needs a free state slot
+    slots = sm.num_free if sm is not None else 0
     for it in self._queue:
       n = self._qlen(it[2])
+      if sm is not None and it[1] == self.shard and not sm.has(it[0]):
+        if slots == 0:  # every slot is held by a live request: wait for one to finish
+          rest.append(it)
+          continue
+        if it[0] not in {b[0] for b in batch}:
+          slots -= 1
       if len(batch) < cap and (not batch or tokens + n <= MAX_STEP_TOKENS):
         batch.append(it)
         tokens += n
@@ -649,7 +657,7 @@ class ShardedInferenceEngine(InferenceEngine):
         apply_ops(self.runner.bm, rid, state.get("pc"))  # the first shard's prefix-cache operations
         x = inp if isinstance(inp, torch.Tensor) else torch.as_tensor(np.asarray(inp))
         L = x.shape[1]
-        xs.append(x.reshape(L, x.shape[2]).to(torch.bfloat16))
+        xs.append(x.reshape(L, x.shape[2]).to(self.runner.hidden_dtype))
       else:  # token ids [1, L]: numpy on the host (no per-request tensor ops; one tensor for the step)
         ids = (inp.detach().cpu().numpy() if isinstance(inp, torch.Tensor) else np.asarray(inp)).reshape(-1)
         if pc is not None and state.get("kv_min"):
@@ -767,6 +775,8 @@ class ShardedInferenceEngine(InferenceEngine):
     repo = registry.get_repo(shard.model_id, "ShardedInferenceEngine")
     if repo is None:
       return None
+    if repo.startswith(registry.LOCAL):  # a model directory given on the command line
+      return Path(repo[len(registry.LOCAL):])
     from ..helpers import xot_home
     p = xot_home() / "downloads" / repo.replace("/", "--")
     return p if (p / "config.json").exists() else None
@@ -778,7 +788,8 @@ class ShardedInferenceEngine(InferenceEngine):
       if self.shard == shard and self.runner is not None:
         return
       model_dir = None
-      if self.shard_downloader is not None and shard.model_id not in registry.SYNTHETIC:
+      local = (registry.get_repo(shard.model_id, "ShardedInferenceEngine") or "").startswith(registry.LOCAL)
+      if self.shard_downloader is not None and shard.model_id not in registry.SYNTHETIC and not local:
         try:
           model_dir = await self.shard_downloader.ensure_shard(shard, "ShardedInferenceEngine")
         except Exception as e:
@@ -811,7 +822,8 @@ class ShardedInferenceEngine(InferenceEngine):
     self.model_path = model_dir
     self.prefix_cache = None
     longrope = (cfg.rope_scaling or {}).get("rope_type") == "longrope"  # the prefix's rotation depends on the total length
-    if PREFIX_CACHE and shard.is_first_layer() and not longrope:
+    # (a cached prefix's pages say nothing about the recurrent state at its end: no reuse for such models)
+    if PREFIX_CACHE and shard.is_first_layer() and not longrope and not cfg.has_state:
       from .prefix_cache import PrefixCache
       self.prefix_cache = PrefixCache(self.runner.bm, int(self.runner.bm.num_blocks * PREFIX_CACHE_FRAC),
                                       single_shard=shard.is_last_layer())

@@ -393,6 +393,9 @@ async def async_main(args, engine=None, device_caps=None):
 
 async def _command(args, node, api, viz) -> int:
   model_name = args.model_name or args.run_model
+  if model_name and os.path.isdir(model_name):  # `xot run DIR`: a local config.json + safetensors
+    from .models.registry import register_local_model
+    register_local_model(model_name)
   if args.command == "run" or args.run_model:
     if not model_name:
       print("Error: model name is required")

@@ -496,6 +496,23 @@ PRESETS: dict[str, ModelConfig] = {
                                   routed_scaling_factor=2.5, topk_method="noaux_tc", n_group=4, topk_group=2,
                                   norm_topk_prob=True, scoring_func="sigmoid"),
 }
+TINY_TAREPEL = {
+  "architecture": "Tarepel", "vocab": 320, "width": 128, "norm": {"eps": 1e-5}, "logit_scale": 0.5,
+  "layers": [
+    {"type": "parallel", "mlp": {"kind": "dense", "ff": 192},
+     "mixer": {"left": {"heads": 4, "kv_heads": 1, "dim": 32, "vdim": 32, "mask": {"size": 48},
+                        "rot": {"base": 10000.0, "dims": 16}, "scale": 0.2},
+               "right": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "conv": 3},
+               "left_scale": 0.7, "right_scale": 0.9}},
+    {"type": "gla", "mlp": None, "mixer": {"heads": 2, "dim": 32, "vdim": 64, "tau": 8.0}},
+    {"type": "gla", "mlp": {"kind": "dense", "ff": 128}, "mixer": {"heads": 4, "dim": 16, "vdim": 32, "tau": 12.0}},
+    {"type": "parallel", "mlp": {"kind": "dense", "ff": 192},
+     "mixer": {"left": {"heads": 2, "kv_heads": 2, "dim": 64, "vdim": 64, "mask": {"size": 32},
+                        "rot": {"base": 50000.0, "dims": 64}, "scale": 0.125},
+               "right": {"heads": 2, "kv_heads": 2, "dim": 32, "vdim": 32, "conv": 4},
+               "left_scale": 1.0, "right_scale": 0.5}},
+  ]}
+PRESETS["tiny-tarepel"] = _tarepel_config(TINY_TAREPEL)
 # aliases of the reference's model cards that share an architecture
 for _alias, _base in {"llama-3.1-70b-bf16": "llama-3.1-70b", "nemotron-70b": "llama-3.1-70b",
                       "deepseek-r1-distill-llama-70b": "llama-3.1-70b", "deepseek-r1-distill-llama-8b": "llama-3.1-8b",

@@ -65,6 +65,7 @@ _CARDS: List[tuple] = [
   ("tiny-deepseek-v2", 3, "synthetic/tiny-deepseek-v2", "Tiny DeepSeek-V2 (synthetic)"),
   ("tiny-deepseek-v3", 3, "synthetic/tiny-deepseek-v3", "Tiny DeepSeek-V3 (synthetic)"),
   ("tiny-llava", 4, "synthetic/tiny-llava", "Tiny LLaVA (synthetic)"),
+  ("tiny-tarepel", 4, "synthetic/tiny-tarepel", "Tiny Tarepel (synthetic)"),
 ]
 
 model_cards: Dict[str, dict] = {mid: {"layers": n, "repo": {ENGINE: repo}} for mid, n, repo, _ in _CARDS}
@@ -72,6 +73,23 @@ SYNTHETIC = {mid for mid, _, repo, _ in _CARDS if repo.startswith("synthetic/")}
 model_cards["dummy"] = {"layers": 8, "repo": {DUMMY: "dummy"}}
 pretty_name: Dict[str, str] = {mid: pretty for mid, _, _, pretty in _CARDS}
 pretty_name["dummy"] = "Dummy"
+
+
+LOCAL = "local:"  # repo prefix of a model served from a directory (register_local_model)
+
+
+def register_local_model(path: str) -> Optional[str]:
+  """A directory with config.json (+ safetensors) becomes a model card whose id is the path as given; its layer
+  count comes from config.json (any architecture models.config.load_config reads).  Returns the id, or None when
+  the path is not such a directory."""
+  import os
+  if not os.path.isfile(os.path.join(path, "config.json")):
+    return None
+  from .config import load_config
+  n = load_config(path).num_layers
+  model_cards[path] = {"layers": n, "repo": {ENGINE: LOCAL + os.path.abspath(path)}}
+  pretty_name[path] = os.path.basename(os.path.normpath(path))
+  return path
 
 
 def get_repo(model_id: str, engine_classname: str) -> Optional[str]:

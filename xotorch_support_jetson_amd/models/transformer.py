@@ -435,7 +435,7 @@ class ShardModel:
     if c.has_state and (self.state is None or inp.state_slots is None):
       raise RuntimeError("a model with recurrent layers needs a state pool and the step's state slots")
     if self.shard.is_first_layer():
-      h = w.embed.index_select(0, x.view(-1).long())
+      h = w.embed.index_select(0, x.view(-1).long().clamp(0, w.embed.shape[0] - 1))
     else:
       h = x.to(torch.float32).contiguous().clone()
     T, D = h.shape
