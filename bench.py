@@ -107,6 +107,84 @@ def gemm_choices(batch: int) -> dict:
   return out
 
 
+MIXER_SIZES = {
+  # width, layers, (attention heads, kv heads, head dim, chunk, rotary dims), recurrence (heads, q/k heads, dim, vdim), ff
+  "1b": dict(width=2048, layers=8, attn=(16, 4, 128, 1024, 64), rec=(16, 8, 128, 128), gla=(16, 64, 128), ff=5632),
+  "3b": dict(width=3072, layers=6, attn=(24, 8, 128, 2048, 128), rec=(24, 8, 128, 128), gla=(24, 64, 128), ff=8192),
+  "8b": dict(width=4096, layers=4, attn=(32, 8, 128, 2048, 64), rec=(32, 16, 128, 128), gla=(32, 64, 128), ff=14336),
+}
+
+
+def mixer_configs(name: str):
+  """(Tarepel-design config, the closest softmax-attention model at equal width / depth / heads / feed-forward)."""
+  from xotorch_support_jetson_amd.models.config import ModelConfig, from_hf_config
+  z = MIXER_SIZES[name]
+  H, G, d, chunk, rot = z["attn"]
+  rh, rg, rd, rdv = z["rec"]
+  gh, gd, gdv = z["gla"]
+  par = {"type": "parallel", "mlp": {"kind": "dense", "ff": z["ff"]},
+         "mixer": {"left": {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "mask": {"size": chunk},
+                            "rot": {"base": 1e6, "dims": rot}, "scale": d ** -0.5},
+                   "right": {"heads": rh, "kv_heads": rg, "dim": rd, "vdim": rdv, "conv": 4},
+                   "left_scale": 1.0, "right_scale": 1.0}}
+  gla = {"type": "gla", "mlp": {"kind": "dense", "ff": z["ff"]}, "mixer": {"heads": gh, "dim": gd, "vdim": gdv, "tau": 16.0}}
+  mixed = from_hf_config({"architecture": "Tarepel", "vocab": 32000, "width": z["width"], "norm": {"eps": 1e-5},
+                          "logit_scale": 1.0, "layers": [par if i % 2 == 0 else gla for i in range(z["layers"])]})
+  dense = ModelConfig("llama", 32000, z["width"], z["ff"], z["layers"], H, G, d, 1e-5, 1e6, None, 32768, False,
+                      bos_token_id=1, eos_token_ids=(2,))
+  return mixed, dense
+
+
+def bench_mixers(args):
+  """Prefill and decode throughput of Tarepel-design layers at sizes like a real model's (random weights), beside
+  the closest existing model (a Llama-style stack of equal width, depth, heads and feed-forward) on the same
+  runner: one prefill step of --mixer-batch prompts of --prompt-len tokens, then HIP-graph decode steps at that
+  context.  One JSON line; not the headline metric."""
+  from xotorch_support_jetson_amd.inference.shard import Shard
+  from xotorch_support_jetson_amd.runtime.runner import ShardRunner
+  dev = torch.device("cuda:0")
+  torch.cuda.set_device(dev)
+  B, L = args.mixer_batch, args.prompt_len
+  res = {}
+  for name in args.mixers.split(","):
+    row = {}
+    for kind, cfg in zip(("tarepel", "llama"), mixer_configs(name)):
+      shard = Shard(f"{kind}-{name}", 0, cfg.num_layers - 1, cfg.num_layers)
+      max_ctx = L + args.warmup + args.steps + 8
+      r = ShardRunner(cfg, shard, dev, num_pages=B * -(-max_ctx // 64) + 4, max_batch=B, max_ctx=max_ctx, seed=0)
+      g = torch.Generator().manual_seed(1)
+      rids = [f"r{i}" for i in range(B)]
+      ids = torch.randint(0, cfg.vocab_size, (B * L,), generator=g, dtype=torch.int32)
+      warm = [f"w{i}" for i in range(B)]  # same shapes once untimed: GEMM choices settle
+      r.forward(warm, [L] * B, ids)
+      for w in warm:
+        r.free(w)
+      sync()
+      t0 = time.perf_counter()
+      logits = r.forward(rids, [L] * B, ids)
+      sync()
+      t_pre = time.perf_counter() - t0
+      tok = logits.argmax(-1).to(torch.int32)
+      for _ in range(args.warmup):
+        tok = r.forward(rids, [1] * B, tok).argmax(-1).to(torch.int32)
+      sync()
+      t0 = time.perf_counter()
+      for _ in range(args.steps):
+        tok = r.forward(rids, [1] * B, tok).argmax(-1).to(torch.int32)
+      sync()
+      t_dec = (time.perf_counter() - t0) / args.steps
+      row[kind] = {"params_m": round(cfg.num_params() / 1e6, 1), "prefill_tok_s": round(B * L / t_pre, 1),
+                   "prefill_ms": round(t_pre * 1e3, 2), "decode_tok_s": round(B / t_dec, 1),
+                   "decode_ms_per_step": round(t_dec * 1e3, 3)}
+      log(f"[mixers {name}] {kind}: {row[kind]}")
+      del r
+      torch.cuda.empty_cache()
+    res[name] = row
+  print(json.dumps({"metric": "prefill / decode tokens/sec of Tarepel-design layers beside a Llama-style stack of equal size",
+                    "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16",
+                    "data": "synthetic prompts, random-init weights", "batch": B, "prompt_len": L, "sizes": res}), flush=True)
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -127,8 +205,14 @@ def main():
   ap.add_argument("--weight-dtype", default="bf16", choices=["bf16", "fp8"],
                   help="fp8: weight-only e4m3 projections (a separate, reduced-precision measurement; the headline "
                        "is bf16)")
+  ap.add_argument("--mixers", default=None, metavar="SIZES",
+                  help="instead of the headline: Tarepel-design layers beside a Llama-style stack at the named sizes "
+                       f"(comma-separated, of {', '.join(MIXER_SIZES)}); one GPU")
+  ap.add_argument("--mixer-batch", type=int, default=16, help="--mixers: sequences per step")
   args = ap.parse_args()
   os.environ["XOT_WEIGHT_DTYPE"] = args.weight_dtype
+  if args.mixers:
+    return bench_mixers(args)
 
   from xotorch_support_jetson_amd.models.config import preset
   from xotorch_support_jetson_amd.parallel.comm import P2PTransport, init_distributed

@@ -93,7 +93,7 @@ def test_chunked_sigmoid_attention(dev, dtype, H, G, d, R, chunk):
   tab = build_cos_sin(R, 256, base, None, dev) if R else torch.zeros(1, 0, device=dev)
   pages = 8
   kc = torch.zeros(pages, G, 64, d, dtype=dtype, device=dev)
-  vc = torch.zeros_like(kc)
+  vc = torch.zeros(pages, G, d, 64, dtype=dtype, device=dev)
   got = [[], []]
   done = [0, 0]
   for new in ([97, 3], [53, 67]):  # two steps; the first request's cut falls inside a page and a chunk
@@ -103,7 +103,8 @@ def test_chunked_sigmoid_attention(dev, dtype, H, G, d, R, chunk):
     q = torch.empty(P.shape[0], H, d, dtype=dtype, device=dev)
     K.rope_kv_store(P, 0, H * d, -1, H, G, d, R, pos, tab, slots, q, kc, vc)
     out = torch.zeros(P.shape[0], H * d + 8, dtype=dtype, device=dev)
-    K.attn_gated_chunk(q, kc, vc, tables, cu, ctx, W["pb"].float().to(dev), scale, chunk, 1.5, out[:, 4:4 + H * d])
+    K.attn_gated_chunk(q, kc, vc, tables, cu, ctx, W["pb"].float().to(dev), scale, chunk, 1.5, out[:, 4:4 + H * d],
+                       max_qlen=max(new))
     for i in range(2):
       got[i].append(out[int(cu[i]):int(cu[i + 1]), 4:4 + H * d])
       done[i] += new[i]

@@ -121,17 +121,32 @@ __global__ void rope_kv_store_k(const float* __restrict__ P, int ldp, int q_off,
       stf(q_out + ((int64_t)t * H + head) * d + i, v);
     } else if (slot >= 0) {
       const int g = head - H;
-      const int64_t o = (((slot / PAGE_TOK) * G + g) * PAGE_TOK + (slot % PAGE_TOK)) * d + i;
-      stf(k_cache + o, v);
-      stf(v_cache + o, v_off >= 0 ? row[v_off + g * d + i] : raw);
+      const int64_t pg = (slot / PAGE_TOK) * G + g;
+      stf(k_cache + (pg * PAGE_TOK + (slot % PAGE_TOK)) * d + i, v);
+      stf(v_cache + (pg * d + i) * PAGE_TOK + (slot % PAGE_TOK), v_off >= 0 ? row[v_off + g * d + i] : raw);
     }
   }
 }
 
 // ------------------------------------------------------------------ chunk-local gated attention
-// One wave per (token, head).  Keys of the query's chunk up to the query: lanes over keys for the scores, then lanes
-// over value dims for the weighted sum.  out[t, h * d + i] = out_scale * sum_j sigmoid(q.k_j * scale + pb[h]) v_j[i].
+// Caches: K [pages, G, 64, d] (a key's dims contiguous), V^T [pages, G, d, 64] (a dim's 64 keys of the page
+// contiguous: the PV product streams 4 / 8 consecutive keys of one dim per load).
+// out[t, h * d + i] = out_scale * sum_j sigmoid(q.k_j * scale + pb[h]) v_j[i] over the keys j <= i's position of
+// the query's chunk.
+//
+// Simple kernel (any d <= 256, bf16 or fp32; single decoded tokens): one wave per (token, head), lanes over keys for
+// the scores, then lanes over value dims for the weighted sum.
 constexpr int ATT_TILE = 512;
+
+__device__ __forceinline__ void ld8(const float* p, float* o) {
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+  o[0] = a[0]; o[1] = a[1]; o[2] = a[2]; o[3] = a[3]; o[4] = b[0]; o[5] = b[1]; o[6] = b[2]; o[7] = b[3];
+}
+__device__ __forceinline__ void ld8(const uint16_t* p, float* o) {
+  const s16x8 a = ld16(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = bf2f(a[i]);
+}
 
 template <typename AT>
 __global__ void attn_gated_chunk_k(const AT* __restrict__ q, const AT* __restrict__ k_cache, const AT* __restrict__ v_cache,
@@ -140,38 +155,56 @@ __global__ void attn_gated_chunk_k(const AT* __restrict__ q, const AT* __restric
                                    int chunk, float out_scale, AT* __restrict__ out, int ldo, int H, int G, int d) {
   extern __shared__ float sm[];
   float* qs = sm;            // [d]
-  float* ws = sm + d;        // [ATT_TILE]
+  float* ws = sm + d;        // [ATT_TILE + 8]: weights of positions a0 .. (a0 = the tile's start rounded down to 8)
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int b = seq_of(cu_q, B, t);
   const int ctx = ctx_lens[b];
   if (ctx <= 0) return;  // padding row of a captured decode batch
   const int pos = ctx - (cu_q[b + 1] - cu_q[b]) + (t - cu_q[b]);
   const int lo = (pos / chunk) * chunk;
-  const int nkeys = pos - lo + 1;
   const int g = h / (H / G);
   for (int i = lane; i < d; i += 64) qs[i] = ldf(q + ((int64_t)t * H + h) * d + i);
   const float bias = pb[h];
   const int* bt = block_tables + (int64_t)b * width;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};  // value dims lane, lane + 64, ... (d <= 256)
-  for (int j0 = 0; j0 < nkeys; j0 += ATT_TILE) {
-    const int nj = min(ATT_TILE, nkeys - j0);
+  for (int p0 = lo; p0 <= pos; p0 += ATT_TILE) {
+    const int p1 = min(p0 + ATT_TILE, pos + 1);  // keys [p0, p1)
+    const int a0 = p0 & ~7, a1 = (p1 + 7) & ~7;  // 8-aligned cover; positions outside [p0, p1) weigh 0
     __syncthreads();
-    for (int j = lane; j < nj; j += 64) {
-      const int p = lo + j0 + j;
-      const AT* kr = k_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * PAGE_TOK + (p % PAGE_TOK)) * d;
-      float s = 0.0f;
-      for (int i = 0; i < d; ++i) s += qs[i] * ldf(kr + i);
-      ws[j] = sigmoidf_(s * scale + bias);
+    for (int p = a0 + lane; p < a1; p += 64) {
+      float w = 0.0f;
+      if (p >= p0 && p < p1) {
+        const AT* kr = k_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * PAGE_TOK + (p % PAGE_TOK)) * d;
+        float s = 0.0f;
+        if (d & 7) {
+          for (int i = 0; i < d; ++i) s += qs[i] * ldf(kr + i);
+        } else {
+          for (int i = 0; i < d; i += 8) {
+            float kv[8];
+            ld8(kr + i, kv);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s += qs[i + e] * kv[e];
+          }
+        }
+        w = sigmoidf_(s * scale + bias);
+      }
+      ws[p - a0] = w;
     }
     __syncthreads();
-    for (int j = 0; j < nj; ++j) {
-      const int p = lo + j0 + j;
-      const AT* vr = v_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * PAGE_TOK + (p % PAGE_TOK)) * d;
-      const float w = ws[j];
+    for (int p = a0; p < a1; p += 8) {  // 8 keys of one page per step
+      const AT* vp = v_cache + ((int64_t)bt[p / PAGE_TOK] * G + g) * d * PAGE_TOK + (p % PAGE_TOK);
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const int i = lane + 64 * c;
-        if (i < d) acc[c] += w * ldf(vr + i);
+        if (i < d) {
+          float vv[8];
+          ld8(vp + (int64_t)i * PAGE_TOK, vv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float w = ws[p - a0 + e];
+            acc[c] += w != 0.0f ? w * vv[e] : 0.0f;  // (a slot no token has written yet may hold anything)
+          }
+        }
       }
     }
   }
@@ -179,6 +212,100 @@ __global__ void attn_gated_chunk_k(const AT* __restrict__ q, const AT* __restric
   for (int c = 0; c < 4; ++c) {
     const int i = lane + 64 * c;
     if (i < d) stf(out + (int64_t)t * ldo + h * d + i, acc[c] * out_scale);
+  }
+}
+
+// MFMA kernel (bf16, d = 32 NK): a wave owns 32 consecutive queries of one (sequence, head) and walks the keys of
+// their chunk(s) 32 at a time.  Scores are computed transposed, S^T = K Q^T (keys x queries), so a lane's four
+// accumulator rows are four consecutive keys of ONE query: after the sigmoid they are, as they lie, the B operand
+// of O^T += V^T P^T, whose k slots (g, j) are read as keys {4g .. 4g+3, 16+4g .. 16+4g+3} on both operands.
+// No LDS, no barriers: K rows and V^T runs come straight from L2.
+template <int NK>
+__global__ __launch_bounds__(256) void attn_gated_chunk_mfma_k(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
+    const float* __restrict__ pb, float scale, int chunk, float out_scale, uint16_t* __restrict__ out, int ldo, int H, int G) {
+  constexpr int D = NK * 32, ND = NK * 2, QT = 2;
+  const int b = blockIdx.x, h = blockIdx.z;
+  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, c = l & 15, g4 = l >> 4;
+  const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0, ctx = ctx_lens[b];
+  const int q0 = (blockIdx.y * 4 + wave) * 32;
+  if (ctx <= 0 || q0 >= qlen) return;
+  const int nq = min(32, qlen - q0);
+  const int pos0 = ctx - qlen + q0;
+  const int gk = h / (H / G);
+  const float bias = pb[h];
+  s16x8 qf[QT][NK];
+  int qpos[QT], qcs[QT];
+  bool qok[QT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int local = qt * 16 + c;
+    qok[qt] = local < nq;
+    qpos[qt] = pos0 + local;
+    qcs[qt] = (qpos[qt] / chunk) * chunk;
+    const uint16_t* qp = q + ((int64_t)(t0 + q0 + local) * H + h) * D + 8 * g4;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) qf[qt][ks] = qok[qt] ? ld16(qp + ks * 32) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+  f32x4 o[QT][ND];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+    for (int db = 0; db < ND; ++db) o[qt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int k_lo = ((pos0 / chunk) * chunk) & ~31, k_hi = pos0 + nq - 1;
+  const int* bt = block_tables + (int64_t)b * width;
+  for (int kb = k_lo; kb <= k_hi; kb += 32) {
+    const int64_t pg = (int64_t)bt[kb >> 6] * G + gk;
+    const int koff = kb & 63;
+    const uint16_t* kp = k_cache + (pg * PAGE_TOK + koff + c) * D + 8 * g4;
+    f32x4 s[2][QT];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) s[kt][qt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        const s16x8 a = ld16(kp + (int64_t)kt * 16 * D + ks * 32);
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) s[kt][qt] = mfma16(a, qf[qt][ks], s[kt][qt]);
+      }
+    s16x8 pf[QT];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int kpos = kb + kt * 16 + 4 * g4 + r;
+          const bool vis = qok[qt] && kpos <= qpos[qt] && kpos >= qcs[qt];
+          const float p = vis ? __fdividef(1.0f, 1.0f + __expf(-(s[kt][qt][r] * scale + bias))) : 0.0f;
+          pf[qt][kt * 4 + r] = (short)f2bf(p);
+        }
+    const uint16_t* vp = v_cache + (pg * D + c) * PAGE_TOK + koff + 4 * g4;
+#pragma unroll
+    for (int db = 0; db < ND; ++db) {
+      const s16x4 v0 = *reinterpret_cast<const s16x4*>(vp + (int64_t)db * 16 * PAGE_TOK);
+      const s16x4 v1 = *reinterpret_cast<const s16x4*>(vp + (int64_t)db * 16 * PAGE_TOK + 16);
+      s16x8 a = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+      // (slots of the page no token has written yet hold zeros or an earlier request's finite values; their weight is 0)
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) o[qt][db] = mfma16(a, pf[qt], o[qt][db]);
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    if (!qok[qt]) continue;
+    uint16_t* op = out + (int64_t)(t0 + q0 + qt * 16 + c) * ldo + h * D + 4 * g4;
+#pragma unroll
+    for (int db = 0; db < ND; ++db) {
+      s16x4 w;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) w[r] = (short)f2bf(o[qt][db][r] * out_scale);
+      *reinterpret_cast<s16x4*>(op + db * 16) = w;
+    }
   }
 }
 
@@ -469,8 +596,9 @@ void rope_kv_store(const at::Tensor& P, int64_t q_off, int64_t k_off, int64_t v_
   MCHECK(k_cache.is_cuda() && k_cache.scalar_type() == q_out.scalar_type() && k_cache.is_contiguous() && k_cache.dim() == 4 &&
              k_cache.size(1) == G && k_cache.size(2) == PAGE_TOK && k_cache.size(3) == d,
          "k_cache must be [pages, G, 64, d] of q_out's dtype");
-  MCHECK(v_cache.is_cuda() && v_cache.scalar_type() == q_out.scalar_type() && v_cache.is_contiguous() &&
-             v_cache.sizes() == k_cache.sizes(), "v_cache must match k_cache");
+  MCHECK(v_cache.is_cuda() && v_cache.scalar_type() == q_out.scalar_type() && v_cache.is_contiguous() && v_cache.dim() == 4 &&
+             v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == G && v_cache.size(2) == d && v_cache.size(3) == PAGE_TOK,
+         "v_cache must be [pages, G, d, 64] of q_out's dtype");
   // positions and slots are checked on the host by their producer (the block manager hands out slots < pages * 64
   // and the runner bounds positions by the table's rows)
   if (q_out.scalar_type() == at::kBFloat16)
@@ -485,17 +613,30 @@ void rope_kv_store(const at::Tensor& P, int64_t q_off, int64_t k_off, int64_t v_
                                                     k_cache.data_ptr<float>(), v_cache.data_ptr<float>());
 }
 
+template <int NK>
+void launch_attn_mfma(dim3 grid, const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache,
+                      const at::Tensor& block_tables, const at::Tensor& cu_q, const at::Tensor& ctx_lens, const at::Tensor& pb,
+                      float scale, int chunk, float out_scale, at::Tensor& out, int ldo, int H, int G) {
+  attn_gated_chunk_mfma_k<NK><<<grid, 256, 0, stream()>>>(
+      (const uint16_t*)q.data_ptr(), (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(),
+      block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(),
+      pb.data_ptr<float>(), scale, chunk, out_scale, (uint16_t*)out.data_ptr(), ldo, H, G);
+}
+
+// max_qlen: the longest run of new tokens of one sequence in this step (1: single decoded tokens -> the wave-per-token
+// kernel; the MFMA kernel takes bf16 with d a multiple of 32).
 void attn_gated_chunk(const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache, const at::Tensor& block_tables,
                       const at::Tensor& cu_q, const at::Tensor& ctx_lens, const at::Tensor& pb, double scale, int64_t chunk,
-                      double out_scale, at::Tensor& out) {
+                      double out_scale, at::Tensor& out, int64_t max_qlen) {
   MCHECK(q.is_cuda() && is_act(q) && q.is_contiguous() && q.dim() == 3, "q must be [T, H, d]");
   const int64_t T = q.size(0), H = q.size(1), d = q.size(2);
   if (T == 0) return;
   MCHECK(k_cache.is_cuda() && k_cache.scalar_type() == q.scalar_type() && k_cache.is_contiguous() && k_cache.dim() == 4 &&
              k_cache.size(2) == PAGE_TOK && k_cache.size(3) == d, "k_cache must be [pages, G, 64, d] of q's dtype");
-  MCHECK(v_cache.is_cuda() && v_cache.scalar_type() == q.scalar_type() && v_cache.is_contiguous() &&
-             v_cache.sizes() == k_cache.sizes(), "v_cache must match k_cache");
   const int64_t G = k_cache.size(1);
+  MCHECK(v_cache.is_cuda() && v_cache.scalar_type() == q.scalar_type() && v_cache.is_contiguous() && v_cache.dim() == 4 &&
+             v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == G && v_cache.size(2) == d && v_cache.size(3) == PAGE_TOK,
+         "v_cache must be [pages, G, d, 64] of q's dtype");
   MCHECK(G > 0 && H % G == 0 && d <= 256 && chunk > 0, "attn_gated_chunk: heads must be a multiple of kv heads, d <= 256");
   i32c(block_tables, "block_tables");
   i32c(cu_q, "cu_q");
@@ -505,9 +646,23 @@ void attn_gated_chunk(const at::Tensor& q, const at::Tensor& k_cache, const at::
   MCHECK(block_tables.dim() == 2 && block_tables.size(0) == B && cu_q.numel() == B + 1 && pb.numel() == H, "batch shape mismatch");
   const int ldo = act_ld(out, T, H * d, "out");
   MCHECK(out.scalar_type() == q.scalar_type(), "out must have q's dtype");
+  const bool bf = q.scalar_type() == at::kBFloat16;
+  if (bf && max_qlen > 1 && d % 32 == 0 && ldo % 4 == 0 && reinterpret_cast<uintptr_t>(out.data_ptr()) % 8 == 0) {
+    const dim3 grid((unsigned)B, (unsigned)((max_qlen + 127) / 128), (unsigned)H);
+#define ATT_CASE(N)                                                                                                         \
+  case N:                                                                                                                   \
+    launch_attn_mfma<N>(grid, q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, (float)scale, (int)chunk, (float)out_scale, \
+                        out, ldo, (int)H, (int)G);                                                                          \
+    break;
+    switch (d / 32) {
+      ATT_CASE(1) ATT_CASE(2) ATT_CASE(3) ATT_CASE(4) ATT_CASE(5) ATT_CASE(6) ATT_CASE(7) ATT_CASE(8)
+    }
+#undef ATT_CASE
+    return;
+  }
   const dim3 grid((unsigned)T, (unsigned)H);
-  const size_t lds = (d + ATT_TILE) * sizeof(float);
-  if (q.scalar_type() == at::kBFloat16)
+  const size_t lds = (d + ATT_TILE + 8) * sizeof(float);
+  if (bf)
     attn_gated_chunk_k<uint16_t><<<grid, 64, lds, stream()>>>(
         (const uint16_t*)q.data_ptr(), (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(),
         block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B,

@@ -95,13 +95,13 @@ class KVCache:
     self.num_pages = num_pages
     self.device = torch.device(device)
     if c.is_mixed:
-      # one K and one V pool per layer that has an attention mixer (None for the others), both [pages, G, 64, d]:
+      # one K [pages, G, 64, d] and one V [pages, G, d, 64] pool per layer that has an attention mixer (None for the others):
       # layers may differ in heads and sizes; the value pool holds whatever the layer's mixer stores as values
       ids = list(layer_ids) if layer_ids is not None else list(range(n_layers))
       specs = [c.layer_specs[i].attn for i in ids]
       self.k = [None if a is None else torch.zeros(num_pages, a.kv_heads, PAGE, a.dim, device=device, dtype=dtype)
                 for a in specs]
-      self.v = [None if a is None else torch.zeros(num_pages, a.kv_heads, PAGE, a.dim, device=device, dtype=dtype)
+      self.v = [None if a is None else torch.zeros(num_pages, a.kv_heads, a.dim, PAGE, device=device, dtype=dtype)
                 for a in specs]
       return
     if c.is_mla:
@@ -397,7 +397,7 @@ class ShardModel:
                     self.kv.k[j], self.kv.v[j])
     off, n = lw.mix_cols["attn"]
     K.attn_gated_chunk(q, self.kv.k[j], self.kv.v[j], inp.block_tables, inp.cu_q, inp.ctx_lens, lw.attn_pb, a.scale,
-                       a.chunk, lw.spec.attn_scale, mix[:, off:off + n])
+                       a.chunk, lw.spec.attn_scale, mix[:, off:off + n], max_qlen=inp.max_qlen)
 
   def _recurrence(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:
     """Linear-attention recurrence over each sequence's state slot (delta rule or per-channel decay), then the
@@ -448,7 +448,7 @@ class ShardModel:
       # activation rows whose K-padding columns stay zero: kernels only write the first `live` columns
       key = (name, live, padded)
       if key not in bufs:
-        bufs[key] = torch.zeros(T, padded, dtype=adt, device=h.device)
+        bufs[key] = (torch.zeros if padded > live else torch.empty)(T, padded, dtype=adt, device=h.device)
       return bufs[key]
     hn = rows("hn", D, -(-D // 128) * 128)
     if n:

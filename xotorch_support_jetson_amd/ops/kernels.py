@@ -458,17 +458,20 @@ def gelu_mul(P, gate_off: int, up_off: int, F: int, out) -> None:
 def rope_kv_store(P, q_off: int, k_off: int, v_off: int, H: int, G: int, d: int, R: int, pos, cos_sin, slots, q_out,
                   k_cache, v_cache) -> None:
   """Rotate-half RoPE on the first R dims of every q / k head (pairs (i, i + R/2)); q -> q_out [T, H, d], the
-  rotated key and the value (v_off < 0: the key before rotation) -> paged caches [pages, G, 64, d] at `slots`."""
+  rotated key -> k_cache [pages, G, 64, d], the value (v_off < 0: the key before rotation) -> v_cache [pages, G, d, 64],
+  both at `slots`."""
   _mix("rope_kv_store", _gpu(P))(P, int(q_off), int(k_off), int(v_off), int(H), int(G), int(d), int(R), pos, cos_sin,
                                  slots, q_out, k_cache, v_cache)
 
 
 def attn_gated_chunk(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, scale: float, chunk: int, out_scale: float,
-                     out) -> None:
+                     out, max_qlen: int = 0) -> None:
   """out [T, H d] = out_scale * sum over the keys j <= i of query i's chunk (floor(i / chunk) == floor(j / chunk))
-  of sigmoid(q_i . k_j * scale + pb[head]) v_j; positions count from each sequence's start."""
+  of sigmoid(q_i . k_j * scale + pb[head]) v_j; positions count from each sequence's start.  Caches: K [pages, G, 64,
+  d], V [pages, G, d, 64].  max_qlen: the step's longest run of new tokens of one sequence (0: unknown -> the total);
+  bf16 steps with runs above one token take the MFMA kernel, single tokens a wave per (token, head)."""
   _mix("attn_gated_chunk", _gpu(q))(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, float(scale), int(chunk),
-                                    float(out_scale), out)
+                                    float(out_scale), out, int(max_qlen) or int(q.shape[0]))
 
 
 def delta_prep(P, x_off: int, b_off: int, a_off: int, conv_w, conv_state, state_slots, cu_q, A_log, dt_bias, H: int,

@@ -269,10 +269,10 @@ def rope_kv_store(P, q_off, k_off, v_off, H, G, d, R, pos, cos_sin, slots, q_out
   ok = slots >= 0
   s = slots[ok].long()
   k_cache[s // PAGE, :, s % PAGE] = rot(k)[ok].to(k_cache.dtype)
-  v_cache[s // PAGE, :, s % PAGE] = v[ok].to(v_cache.dtype)
+  v_cache[s // PAGE, :, :, s % PAGE] = v[ok].to(v_cache.dtype)
 
 
-def attn_gated_chunk(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, scale, chunk, out_scale, out):
+def attn_gated_chunk(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, scale, chunk, out_scale, out, max_qlen=0):
   T, H, d = q.shape
   G = k_cache.shape[1]
   for b in range(ctx_lens.numel()):
@@ -282,7 +282,7 @@ def attn_gated_chunk(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, scal
     npg = -(-n // PAGE)
     pages = block_tables[b, :npg].long()
     k = k_cache[pages].permute(0, 2, 1, 3).reshape(npg * PAGE, G, d)[:n].float().repeat_interleave(H // G, 1)
-    v = v_cache[pages].permute(0, 2, 1, 3).reshape(npg * PAGE, G, d)[:n].float().repeat_interleave(H // G, 1)
+    v = v_cache[pages].permute(0, 3, 1, 2).reshape(npg * PAGE, G, d)[:n].float().repeat_interleave(H // G, 1)
     qpos = torch.arange(n - (t1 - t0), n)[:, None]
     kpos = torch.arange(n)[None, :]
     vis = (kpos <= qpos) & (kpos // chunk == qpos // chunk)
