@@ -137,7 +137,7 @@ def test_gated_delta_rule(dev, dtype, H, G, d, dv, taps):
     want.append(torch.stack([O.gated_delta_rule(W, "", m, h[p], mem, eps) for p in range(h.shape[0])]))
   f = lambda t: t.float().to(dev)
   conv_w = f(torch.cat([W["q.conv"], W["k.conv"], W["v.conv"]]))
-  state = torch.full((3, H, d, dv), 7.0, device=dev)
+  state = torch.full((3, H, dv, d), 7.0, device=dev)
   conv_state = torch.full((3, taps - 1, C), 7.0, device=dev)
   for s in (2, 0):  # the slots these sequences get, cleared as on admission
     state[s].zero_()
@@ -178,7 +178,7 @@ def test_gated_linear_attention(dev, dtype, H, d, dv, rank, tau):
     mem = {}
     want.append(torch.stack([O.gated_linear_attention(W, "", m, h[p], mem, eps) for p in range(h.shape[0])]))
   f = lambda t: t.float().to(dev)
-  state = torch.zeros(2, H, d, dv, device=dev)
+  state = torch.zeros(2, H, dv, d, device=dev)
   got, done = [[], []], [0, 0]
   for new in ([17, 1], [1, 30], [42, 2]):
     cu, slots = _slots_batch(new, [1, 0], dev)

@@ -390,11 +390,20 @@ __global__ void gla_prep_k(const float* __restrict__ P, int ldp, int a1_off, int
 }
 
 // ------------------------------------------------------------------ the recurrence
-// Workgroup = (sequence, value head, block of 64 value channels); 256 threads = 64 columns x 4 row groups, the row
-// group in the low lane bits so the two dot products reduce over lanes l ^ 1, l ^ 2.  A thread keeps rows
-// rg + 4 m (m < KR) of its column in registers.  Tokens are staged through LDS REC_TB at a time.
+// State in memory: S^T [slots, H, dv, d] (a value channel's d key rows contiguous).
+// Workgroup = (sequence, value head, 16 value channels); 256 threads = 16 channels x 16 row groups, the row group in
+// the low lane bits: the two dot products reduce inside 16-lane rows (lanes l ^ 1, 2, 4, 8).  A thread keeps the KR
+// consecutive key rows rg KR .. rg KR + KR - 1 of its channel in registers (d <= 16 KR), so state loads and stores
+// are contiguous runs and a token's k / q slices are vector LDS reads.  Tokens are staged through LDS REC_TB at a time.
 // DELTA: S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q.   else: S = diag(a) S + k v^T; o = S^T q.
 constexpr int REC_TB = 16;
+constexpr int REC_COLS = 16;
+
+__device__ __forceinline__ float row16_sum(float v) {
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
 
 template <int KR, bool DELTA>
 __global__ __launch_bounds__(256) void linear_recurrence_k(
@@ -402,22 +411,20 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
     const float* __restrict__ decay, const float* __restrict__ beta, float q_scale, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_q, int H, int G, int d, int dv,
     float* __restrict__ out) {
-  constexpr int DP = KR * 4;  // padded key dim
-  __shared__ float sq[REC_TB][DP], sk[REC_TB][DP], sa[REC_TB][DELTA ? 1 : DP], sv[REC_TB][64], sg[REC_TB][2];
+  constexpr int DP = KR * 16;  // padded key dim
+  __shared__ __attribute__((aligned(16))) float sq[REC_TB][DP], sk[REC_TB][DP], sa[REC_TB][DELTA ? 4 : DP];
+  __shared__ float sv[REC_TB][REC_COLS], sg[REC_TB][2];
   const int b = blockIdx.x, h = blockIdx.y, cb = blockIdx.z;
   const int slot = state_slots[b];
   const int t0 = cu_q[b], n = cu_q[b + 1] - t0;
   if (slot < 0 || n <= 0) return;
-  const int tid = threadIdx.x, rg = tid & 3, col = cb * 64 + (tid >> 2);
+  const int tid = threadIdx.x, rg = tid & 15, cl = tid >> 4, col = cb * REC_COLS + cl;
   const bool live = col < dv;
   const int hk = h / (H / G);
-  float* S = state + (((int64_t)slot * H + h) * d) * dv;
+  float* S = state + (((int64_t)slot * H + h) * dv + (live ? col : 0)) * d + rg * KR;
   float s[KR];
 #pragma unroll
-  for (int m = 0; m < KR; ++m) {
-    const int i = rg + 4 * m;
-    s[m] = (live && i < d) ? S[(int64_t)i * dv + col] : 0.0f;
-  }
+  for (int m = 0; m < KR; ++m) s[m] = (live && rg * KR + m < d) ? S[m] : 0.0f;
   for (int tb = 0; tb < n; tb += REC_TB) {
     const int nt = min(REC_TB, n - tb);
     __syncthreads();
@@ -429,9 +436,9 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
       sk[tt][i] = in ? k[t * ldk + hk * d + i] : 0.0f;
       if (!DELTA) sa[tt][i] = in ? decay[(t * H + h) * d + i] : 0.0f;
     }
-    for (int e = tid; e < nt * 64; e += 256) {
-      const int tt = e >> 6, c = cb * 64 + (e & 63);
-      sv[tt][e & 63] = c < dv ? v[(int64_t)(t0 + tb + tt) * ldv + h * dv + c] : 0.0f;
+    for (int e = tid; e < nt * REC_COLS; e += 256) {
+      const int tt = e / REC_COLS, c = cb * REC_COLS + (e % REC_COLS);
+      sv[tt][e % REC_COLS] = c < dv ? v[(int64_t)(t0 + tb + tt) * ldv + h * dv + c] : 0.0f;
     }
     if (DELTA && tid < nt) {
       sg[tid][0] = decay[(int64_t)(t0 + tb + tid) * H + h];
@@ -439,42 +446,43 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
-      const float vc = sv[tt][tid >> 2];
-      float o = 0.0f;
+      const float vc = sv[tt][cl];
+      float kk[KR], qq[KR];
+#pragma unroll
+      for (int m = 0; m < KR; ++m) {
+        kk[m] = sk[tt][rg * KR + m];
+        qq[m] = sq[tt][rg * KR + m];
+      }
+      float o0 = 0.0f, o1 = 0.0f;
       if (DELTA) {
         const float g = sg[tt][0], bt = sg[tt][1];
-        float dot = 0.0f;
+        float d0 = 0.0f, d1 = 0.0f;
 #pragma unroll
         for (int m = 0; m < KR; ++m) {
           s[m] *= g;
-          dot += s[m] * sk[tt][rg + 4 * m];
+          if (m & 1) d1 += s[m] * kk[m]; else d0 += s[m] * kk[m];
         }
-        dot += __shfl_xor(dot, 1, 64);
-        dot += __shfl_xor(dot, 2, 64);
-        const float u = bt * (vc - dot);
+        const float u = bt * (vc - row16_sum(d0 + d1));
 #pragma unroll
         for (int m = 0; m < KR; ++m) {
-          s[m] += sk[tt][rg + 4 * m] * u;
-          o += s[m] * sq[tt][rg + 4 * m];
+          s[m] += kk[m] * u;
+          if (m & 1) o1 += s[m] * qq[m]; else o0 += s[m] * qq[m];
         }
       } else {
 #pragma unroll
         for (int m = 0; m < KR; ++m) {
-          s[m] = sa[tt][rg + 4 * m] * s[m] + sk[tt][rg + 4 * m] * vc;
-          o += s[m] * sq[tt][rg + 4 * m];
+          s[m] = sa[tt][rg * KR + m] * s[m] + kk[m] * vc;
+          if (m & 1) o1 += s[m] * qq[m]; else o0 += s[m] * qq[m];
         }
       }
-      o += __shfl_xor(o, 1, 64);
-      o += __shfl_xor(o, 2, 64);
+      const float o = row16_sum(o0 + o1);
       if (live && rg == 0) out[(int64_t)(t0 + tb + tt) * H * dv + h * dv + col] = o;
     }
   }
   if (live) {
 #pragma unroll
-    for (int m = 0; m < KR; ++m) {
-      const int i = rg + 4 * m;
-      if (i < d) S[(int64_t)i * dv + col] = s[m];
-    }
+    for (int m = 0; m < KR; ++m)
+      if (rg * KR + m < d) S[m] = s[m];
   }
 }
 
@@ -739,11 +747,11 @@ void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int 
                                                               cu, H, G, d, dv, out);                                     \
     break;
   switch (KR) {
+    REC_CASE(1)
+    REC_CASE(2)
     REC_CASE(4)
     REC_CASE(8)
     REC_CASE(16)
-    REC_CASE(32)
-    REC_CASE(64)
     default:
       MCHECK(false, "linear_recurrence: key dim above 256");
   }
@@ -751,7 +759,7 @@ void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int 
 }
 
 // q / k [T, G d], v [T, H dv]: fp32 rows of unit inner stride (column slices allowed).  decay [T, H] (delta) or
-// [T, H d] (per key channel); beta [T, H] (delta only).  state [slots, H, d, dv].
+// [T, H d] (per key channel); beta [T, H] (delta only).  state [slots, H, dv, d] (S^T: key rows contiguous).
 void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& decay,
                        const c10::optional<at::Tensor>& beta, double q_scale, at::Tensor& state, const at::Tensor& state_slots,
                        const at::Tensor& cu_q, at::Tensor& out) {
@@ -761,8 +769,8 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   f32c(out, "out");
   i32c(state_slots, "state_slots");
   i32c(cu_q, "cu_q");
-  MCHECK(state.dim() == 4, "state must be [slots, H, d, dv]");
-  const int64_t T = q.size(0), H = state.size(1), d = state.size(2), dv = state.size(3), B = state_slots.numel();
+  MCHECK(state.dim() == 4, "state must be [slots, H, dv, d]");
+  const int64_t T = q.size(0), H = state.size(1), dv = state.size(2), d = state.size(3), B = state_slots.numel();
   if (T == 0 || B == 0) return;
   MCHECK(q.size(1) % d == 0 && q.size(1) == k.size(1), "q / k must be [T, G d]");
   const int64_t G = q.size(1) / d;
@@ -776,9 +784,9 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   } else {
     MCHECK(decay.numel() == T * H * d && G == H, "per-channel decay must be [T, H d] with one q / k head per value head");
   }
-  int KR = 4;
-  while (KR * 4 < d) KR *= 2;
-  const dim3 grid((unsigned)B, (unsigned)H, (unsigned)((dv + 63) / 64));
+  int KR = 1;
+  while (KR * 16 < d) KR *= 2;
+  const dim3 grid((unsigned)B, (unsigned)H, (unsigned)((dv + REC_COLS - 1) / REC_COLS));
   if (delta)
     launch_rec<true>(KR, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,
                      decay.data_ptr<float>(), beta->data_ptr<float>(), (float)q_scale, state.data_ptr<float>(),

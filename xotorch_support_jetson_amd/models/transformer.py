@@ -128,7 +128,7 @@ class KVCache:
 
 class StatePool:
   """Recurrent state of a shard's layers, one slot per live request (models.config.LinearRecurrenceSpec): per layer
-  with a recurrence S [slots, H, d, dv] fp32 and, for rules with short convolutions, the last taps - 1 convolution
+  with a recurrence S^T [slots, H, dv, d] fp32 (a value channel's key rows contiguous) and, for rules with short convolutions, the last taps - 1 convolution
   inputs [slots, taps - 1, channels] fp32.  A slot is cleared when a request is admitted to it."""
 
   def __init__(self, c: ModelConfig, layer_ids, slots: int, device):
@@ -137,7 +137,7 @@ class StatePool:
     self.conv: List[Optional[torch.Tensor]] = []
     for i in layer_ids:
       r = c.layer_specs[i].rec
-      self.S.append(None if r is None else torch.zeros(slots, r.heads, r.dim, r.vdim, device=device, dtype=torch.float32))
+      self.S.append(None if r is None else torch.zeros(slots, r.heads, r.vdim, r.dim, device=device, dtype=torch.float32))
       ch = 0 if r is None or r.conv <= 0 else 2 * r.kv_heads * r.dim + r.heads * r.vdim
       self.conv.append(torch.zeros(slots, max(r.conv - 1, 0), ch, device=device, dtype=torch.float32) if ch else None)
 

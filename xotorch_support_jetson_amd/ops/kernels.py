@@ -487,7 +487,7 @@ def gla_prep(P, a1_off: int, a2, a2_b, tau: float, decay) -> None:
 
 
 def linear_recurrence(q, k, v, decay, beta, q_scale: float, state, state_slots, cu_q, out) -> None:
-  """Per sequence and value head, token by token on the fp32 state [slots, H, d, dv] (updated in place):
+  """Per sequence and value head, token by token on the fp32 state, stored S^T [slots, H, dv, d] (updated in place):
   beta given (delta rule, decay [T, H]):  S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q
   else (decay [T, H d] per key channel):  S = diag(a) S + k v^T; o = S^T q.      q is scaled by q_scale."""
   _mix("linear_recurrence", _gpu(q))(q, k, v, decay, beta, float(q_scale), state, state_slots, cu_q, out)

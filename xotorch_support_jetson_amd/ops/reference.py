@@ -317,14 +317,14 @@ def gla_prep(P, a1_off, a2, a2_b, tau, decay):
 
 
 def linear_recurrence(q, k, v, decay, beta, q_scale, state, state_slots, cu_q, out):
-  _, H, d, dv = state.shape
+  _, H, dv, d = state.shape  # stored transposed: S^T [dv, d] per head
   G = q.shape[1] // d
   rep = H // G
   for b in range(state_slots.numel()):
     t0, t1, slot = int(cu_q[b]), int(cu_q[b + 1]), int(state_slots[b])
     if slot < 0 or t1 == t0:
       continue
-    S = state[slot]
+    S = state[slot].transpose(1, 2)  # [H, d, dv] view; updates land in the slot
     for t in range(t0, t1):
       qt = (q[t].float() * q_scale).reshape(G, d).repeat_interleave(rep, 0)
       kt = k[t].float().reshape(G, d).repeat_interleave(rep, 0)
