@@ -215,89 +215,127 @@ __global__ void attn_gated_chunk_k(const AT* __restrict__ q, const AT* __restric
   }
 }
 
-// MFMA kernel (bf16, d = 32 NK): a wave owns 32 consecutive queries of one (sequence, head) and walks the keys of
-// their chunk(s) 32 at a time.  Scores are computed transposed, S^T = K Q^T (keys x queries), so a lane's four
-// accumulator rows are four consecutive keys of ONE query: after the sigmoid they are, as they lie, the B operand
-// of O^T += V^T P^T, whose k slots (g, j) are read as keys {4g .. 4g+3, 16+4g .. 16+4g+3} on both operands.
-// No LDS, no barriers: K rows and V^T runs come straight from L2.
+// MFMA kernel (bf16, d = 32 NK): a workgroup owns 128 consecutive queries of one (sequence, head), 32 per wave, and
+// walks the keys of their chunk(s) a tile of KT keys at a time: the K rows and V^T runs of the tile are staged in LDS
+// with whole-line loads and shared by the four waves.  Scores are computed transposed, S^T = K Q^T (keys x queries),
+// so a lane's four accumulator rows are four consecutive keys of ONE query: after the sigmoid they are, as they lie,
+// the B operand of O^T += V^T P^T, whose k slots (g, j) are read as keys {4g .. 4g+3, 16+4g .. 16+4g+3} on both
+// operands.  LDS rows are padded by 16 B so the fragment reads of 16 rows hit distinct banks.
 template <int NK>
 __global__ __launch_bounds__(256) void attn_gated_chunk_mfma_k(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
     const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
     const float* __restrict__ pb, float scale, int chunk, float out_scale, uint16_t* __restrict__ out, int ldo, int H, int G) {
   constexpr int D = NK * 32, ND = NK * 2, QT = 2;
+  constexpr int KT = D > 192 ? 32 : 64;  // keys per tile (a page holds a whole number of tiles)
+  constexpr int KP = D + 8, VP = KT + 8;
+  __shared__ __attribute__((aligned(16))) uint16_t sK[KT][KP], sV[D][VP];
   const int b = blockIdx.x, h = blockIdx.z;
   const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, c = l & 15, g4 = l >> 4;
   const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0, ctx = ctx_lens[b];
-  const int q0 = (blockIdx.y * 4 + wave) * 32;
-  if (ctx <= 0 || q0 >= qlen) return;
-  const int nq = min(32, qlen - q0);
-  const int pos0 = ctx - qlen + q0;
+  const int wq0 = blockIdx.y * 128;
+  if (ctx <= 0 || wq0 >= qlen) return;
+  const int q0 = wq0 + wave * 32;
+  const bool active = q0 < qlen;
+  const int nq = active ? min(32, qlen - q0) : 0;
+  const int pos0 = ctx - qlen + q0;  // position of the wave's first query
   const int gk = h / (H / G);
   const float bias = pb[h];
   s16x8 qf[QT][NK];
   int qpos[QT], qcs[QT];
-  bool qok[QT];
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     const int local = qt * 16 + c;
-    qok[qt] = local < nq;
+    const bool ok = local < nq;
     qpos[qt] = pos0 + local;
     qcs[qt] = (qpos[qt] / chunk) * chunk;
     const uint16_t* qp = q + ((int64_t)(t0 + q0 + local) * H + h) * D + 8 * g4;
 #pragma unroll
-    for (int ks = 0; ks < NK; ++ks) qf[qt][ks] = qok[qt] ? ld16(qp + ks * 32) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    for (int ks = 0; ks < NK; ++ks) qf[qt][ks] = ok ? ld16(qp + ks * 32) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
   }
   f32x4 o[QT][ND];
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
     for (int db = 0; db < ND; ++db) o[qt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int k_lo = ((pos0 / chunk) * chunk) & ~31, k_hi = pos0 + nq - 1;
+  // the wave's keys [k_lo, k_hi]; the workgroup's tiles cover the union over its waves
+  const int k_lo = active ? (pos0 / chunk) * chunk : 0x7fffffff, k_hi = active ? pos0 + nq - 1 : -1;
+  const int cs_last = active ? (k_hi / chunk) * chunk : 0;  // a block at or after it and wholly before pos0 needs no mask
+  const int wpos0 = ctx - qlen + wq0;
+  const int t_lo = ((wpos0 / chunk) * chunk) & ~(KT - 1), t_hi = wpos0 + min(128, qlen - wq0) - 1;
   const int* bt = block_tables + (int64_t)b * width;
-  for (int kb = k_lo; kb <= k_hi; kb += 32) {
-    const int64_t pg = (int64_t)bt[kb >> 6] * G + gk;
-    const int koff = kb & 63;
-    const uint16_t* kp = k_cache + (pg * PAGE_TOK + koff + c) * D + 8 * g4;
-    f32x4 s[2][QT];
+  // sigmoid(s scale + bias) = 1 / (1 + 2^(s ea + eb))
+  const float ea = -scale * 1.4426950408889634f, eb = -bias * 1.4426950408889634f;
+  for (int tb = t_lo; tb <= t_hi; tb += KT) {
+    const int64_t pg = (int64_t)bt[tb >> 6] * G + gk;
+    const int koff = tb & 63;
+    __syncthreads();  // the previous tile has been consumed
+    for (int ch = threadIdx.x; ch < KT * (D / 8); ch += 256) {
+      const int row = ch / (D / 8), cc = ch - row * (D / 8);
+      st16(&sK[row][cc * 8], ld16(k_cache + ((pg * PAGE_TOK) + koff + row) * D + cc * 8));
+    }
+    for (int ch = threadIdx.x; ch < D * (KT / 8); ch += 256) {
+      const int row = ch / (KT / 8), cc = ch - row * (KT / 8);
+      st16(&sV[row][cc * 8], ld16(v_cache + (pg * D + row) * PAGE_TOK + koff + cc * 8));
+    }
+    __syncthreads();
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int qt = 0; qt < QT; ++qt) s[kt][qt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < NK; ++ks)
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-        const s16x8 a = ld16(kp + (int64_t)kt * 16 * D + ks * 32);
-#pragma unroll
-        for (int qt = 0; qt < QT; ++qt) s[kt][qt] = mfma16(a, qf[qt][ks], s[kt][qt]);
-      }
-    s16x8 pf[QT];
-#pragma unroll
-    for (int qt = 0; qt < QT; ++qt)
+    for (int sub = 0; sub < KT / 32; ++sub) {
+      const int kb = tb + sub * 32;
+      if (kb > k_hi || kb + 31 < k_lo) continue;  // (wave-uniform) none of these keys is visible to this wave
+      f32x4 s[2][QT];
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int kpos = kb + kt * 16 + 4 * g4 + r;
-          const bool vis = qok[qt] && kpos <= qpos[qt] && kpos >= qcs[qt];
-          const float p = vis ? __fdividef(1.0f, 1.0f + __expf(-(s[kt][qt][r] * scale + bias))) : 0.0f;
-          pf[qt][kt * 4 + r] = (short)f2bf(p);
-        }
-    const uint16_t* vp = v_cache + (pg * D + c) * PAGE_TOK + koff + 4 * g4;
+        for (int qt = 0; qt < QT; ++qt) s[kt][qt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int db = 0; db < ND; ++db) {
-      const s16x4 v0 = *reinterpret_cast<const s16x4*>(vp + (int64_t)db * 16 * PAGE_TOK);
-      const s16x4 v1 = *reinterpret_cast<const s16x4*>(vp + (int64_t)db * 16 * PAGE_TOK + 16);
-      s16x8 a = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+      for (int ks = 0; ks < NK; ++ks)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+          const s16x8 a = ld16(&sK[sub * 32 + kt * 16 + c][ks * 32 + 8 * g4]);
+#pragma unroll
+          for (int qt = 0; qt < QT; ++qt) s[kt][qt] = mfma16(a, qf[qt][ks], s[kt][qt]);
+        }
+      const bool full = kb + 31 <= pos0 && kb >= cs_last;  // every key of the block is visible to every query
+      s16x8 pf[QT];
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        u32x4 packed;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int r2 = 0; r2 < 2; ++r2) {
+            float pr[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              const int r = 2 * r2 + e;
+              float p = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(s[kt][qt][r] * ea + eb));
+              if (!full) {
+                const int kpos = kb + kt * 16 + 4 * g4 + r;
+                p = (kpos <= qpos[qt] && kpos >= qcs[qt]) ? p : 0.0f;
+              }
+              pr[e] = p;
+            }
+            // two bf16 (rounded half up: the weights are positive and finite) in one dword
+            packed[kt * 2 + r2] = __builtin_amdgcn_perm(__float_as_uint(pr[1]) + 0x8000u, __float_as_uint(pr[0]) + 0x8000u,
+                                                        0x07060302u);
+          }
+        pf[qt] = __builtin_bit_cast(s16x8, packed);
+      }
       // (slots of the page no token has written yet hold zeros or an earlier request's finite values; their weight is 0)
 #pragma unroll
-      for (int qt = 0; qt < QT; ++qt) o[qt][db] = mfma16(a, pf[qt], o[qt][db]);
+      for (int db = 0; db < ND; ++db) {
+        const s16x4 v0 = *reinterpret_cast<const s16x4*>(&sV[db * 16 + c][sub * 32 + 4 * g4]);
+        const s16x4 v1 = *reinterpret_cast<const s16x4*>(&sV[db * 16 + c][sub * 32 + 16 + 4 * g4]);
+        const s16x8 a = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) o[qt][db] = mfma16(a, pf[qt], o[qt][db]);
+      }
     }
   }
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
-    if (!qok[qt]) continue;
+    if (qt * 16 + c >= nq) continue;
     uint16_t* op = out + (int64_t)(t0 + q0 + qt * 16 + c) * ldo + h * D + 4 * g4;
 #pragma unroll
     for (int db = 0; db < ND; ++db) {
@@ -391,93 +429,142 @@ __global__ void gla_prep_k(const float* __restrict__ P, int ldp, int a1_off, int
 
 // ------------------------------------------------------------------ the recurrence
 // State in memory: S^T [slots, H, dv, d] (a value channel's d key rows contiguous).
-// Workgroup = (sequence, value head, 16 value channels); 256 threads = 16 channels x 16 row groups, the row group in
-// the low lane bits: the two dot products reduce inside 16-lane rows (lanes l ^ 1, 2, 4, 8).  A thread keeps the KR
-// consecutive key rows rg KR .. rg KR + KR - 1 of its channel in registers (d <= 16 KR), so state loads and stores
-// are contiguous runs and a token's k / q slices are vector LDS reads.  Tokens are staged through LDS REC_TB at a time.
+// Workgroup = (sequence, value head, 256 / RS value channels); 256 threads = channels x RS row groups, the row group
+// in the low lane bits: the two dot products reduce inside DPP rows, register to register.  A thread keeps the KR
+// consecutive key rows rg KR .. rg KR + KR - 1 of its channel in registers (d <= RS KR), so state loads and stores are
+// contiguous runs and a token's k / q slices are vector LDS reads.  RS = 4 does the least work per state element (the
+// choice when sequences x heads x channels fill the chip); RS = 16 spreads one (sequence, head) over four times the
+// lanes.  Tokens are staged through LDS TB at a time, double-buffered: the next block's global loads are in flight
+// while the current one is consumed.
 // DELTA: S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q.   else: S = diag(a) S + k v^T; o = S^T q.
-constexpr int REC_TB = 16;
-constexpr int REC_COLS = 16;
-
-__device__ __forceinline__ float row16_sum(float v) {
-#pragma unroll
-  for (int o = 1; o < 16; o <<= 1) v += __shfl_xor(v, o, 64);
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int m = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
+  return v + __int_as_float(m);
+}
+// sum over RS adjacent lanes, result in each of them: lanes ^1 and ^2 by quad permutes, then (RS 16) the mirrored
+// half row and the mirrored row, whose lanes already hold equal quad / half-row sums
+template <int RS>
+__device__ __forceinline__ float group_sum(float v) {
+  v = dpp_add<0xB1>(v);  // quad_perm [1, 0, 3, 2]
+  v = dpp_add<0x4E>(v);  // quad_perm [2, 3, 0, 1]
+  if (RS == 16) {
+    v = dpp_add<0x141>(v);  // row_half_mirror
+    v = dpp_add<0x140>(v);  // row_mirror
+  }
   return v;
 }
 
-template <int KR, bool DELTA>
+template <int KR, int RS, bool DELTA>
 __global__ __launch_bounds__(256) void linear_recurrence_k(
     const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
     const float* __restrict__ decay, const float* __restrict__ beta, float q_scale, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_q, int H, int G, int d, int dv,
     float* __restrict__ out) {
-  constexpr int DP = KR * 16;  // padded key dim
-  __shared__ __attribute__((aligned(16))) float sq[REC_TB][DP], sk[REC_TB][DP], sa[REC_TB][DELTA ? 4 : DP];
-  __shared__ float sv[REC_TB][REC_COLS], sg[REC_TB][2];
+  constexpr int DP = KR * RS;  // padded key dim
+  constexpr int COLS = 256 / RS;
+  constexpr int TB = DP >= 256 ? 8 : 16;
+  constexpr int NQ = TB * DP / 256, NV = (TB * COLS + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float sq[2][TB][DP], sk[2][TB][DP], sa[2][TB][DELTA ? 4 : DP];
+  __shared__ float sv[2][TB][COLS], sg[2][TB][2];
   const int b = blockIdx.x, h = blockIdx.y, cb = blockIdx.z;
   const int slot = state_slots[b];
   const int t0 = cu_q[b], n = cu_q[b + 1] - t0;
   if (slot < 0 || n <= 0) return;
-  const int tid = threadIdx.x, rg = tid & 15, cl = tid >> 4, col = cb * REC_COLS + cl;
+  const int tid = threadIdx.x, rg = tid % RS, cl = tid / RS, col = cb * COLS + cl;
   const bool live = col < dv;
   const int hk = h / (H / G);
   float* S = state + (((int64_t)slot * H + h) * dv + (live ? col : 0)) * d + rg * KR;
   float s[KR];
 #pragma unroll
   for (int m = 0; m < KR; ++m) s[m] = (live && rg * KR + m < d) ? S[m] : 0.0f;
-  for (int tb = 0; tb < n; tb += REC_TB) {
-    const int nt = min(REC_TB, n - tb);
-    __syncthreads();
-    for (int e = tid; e < nt * DP; e += 256) {
-      const int tt = e / DP, i = e - tt * DP;
+
+  float pq[NQ], pk[NQ], pa[DELTA ? 1 : NQ], pv[NV], pg0 = 0.0f, pg1 = 0.0f;
+  auto fetch = [&](int tb) {  // global -> registers: tokens tb .. tb + TB - 1 of the sequence (zeros past its end)
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {
+      const int e = tid + 256 * j, tt = e / DP, i = e - tt * DP;
       const int64_t t = t0 + tb + tt;
-      const bool in = i < d;
-      sq[tt][i] = in ? q[t * ldq + hk * d + i] * q_scale : 0.0f;
-      sk[tt][i] = in ? k[t * ldk + hk * d + i] : 0.0f;
-      if (!DELTA) sa[tt][i] = in ? decay[(t * H + h) * d + i] : 0.0f;
+      const bool in = i < d && tb + tt < n;
+      pq[j] = in ? q[t * ldq + hk * d + i] * q_scale : 0.0f;
+      pk[j] = in ? k[t * ldk + hk * d + i] : 0.0f;
+      if (!DELTA) pa[j] = in ? decay[(t * H + h) * d + i] : 0.0f;
     }
-    for (int e = tid; e < nt * REC_COLS; e += 256) {
-      const int tt = e / REC_COLS, c = cb * REC_COLS + (e % REC_COLS);
-      sv[tt][e % REC_COLS] = c < dv ? v[(int64_t)(t0 + tb + tt) * ldv + h * dv + c] : 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int e = tid + 256 * j, tt = e / COLS, c = cb * COLS + e % COLS;
+      pv[j] = (e < TB * COLS && c < dv && tb + tt < n) ? v[(int64_t)(t0 + tb + tt) * ldv + h * dv + c] : 0.0f;
     }
-    if (DELTA && tid < nt) {
-      sg[tid][0] = decay[(int64_t)(t0 + tb + tid) * H + h];
-      sg[tid][1] = beta[(int64_t)(t0 + tb + tid) * H + h];
+    if (DELTA && tid < TB && tb + tid < n) {
+      pg0 = decay[(int64_t)(t0 + tb + tid) * H + h];
+      pg1 = beta[(int64_t)(t0 + tb + tid) * H + h];
     }
-    __syncthreads();
+  };
+  auto stage = [&](int buf) {  // registers -> LDS
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {
+      const int e = tid + 256 * j, tt = e / DP, i = e - tt * DP;
+      sq[buf][tt][i] = pq[j];
+      sk[buf][tt][i] = pk[j];
+      if (!DELTA) sa[buf][tt][i] = pa[j];
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int e = tid + 256 * j;
+      if (e < TB * COLS) sv[buf][e / COLS][e % COLS] = pv[j];
+    }
+    if (DELTA && tid < TB) {
+      sg[buf][tid][0] = pg0;
+      sg[buf][tid][1] = pg1;
+    }
+  };
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  int buf = 0;
+  for (int tb = 0; tb < n; tb += TB, buf ^= 1) {
+    const int nt = min(TB, n - tb);
+    const bool more = tb + TB < n;
+    if (more) fetch(tb + TB);
+#pragma unroll 2
     for (int tt = 0; tt < nt; ++tt) {
-      const float vc = sv[tt][cl];
+      const float vc = sv[buf][tt][cl];
       float kk[KR], qq[KR];
 #pragma unroll
       for (int m = 0; m < KR; ++m) {
-        kk[m] = sk[tt][rg * KR + m];
-        qq[m] = sq[tt][rg * KR + m];
+        kk[m] = sk[buf][tt][rg * KR + m];
+        qq[m] = sq[buf][tt][rg * KR + m];
       }
-      float o0 = 0.0f, o1 = 0.0f;
+      float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
       if (DELTA) {
-        const float g = sg[tt][0], bt = sg[tt][1];
-        float d0 = 0.0f, d1 = 0.0f;
+        const float g = sg[buf][tt][0], bt = sg[buf][tt][1];
+        float d0 = 0.0f, d1 = 0.0f, d2 = 0.0f, d3 = 0.0f;
 #pragma unroll
         for (int m = 0; m < KR; ++m) {
           s[m] *= g;
-          if (m & 1) d1 += s[m] * kk[m]; else d0 += s[m] * kk[m];
+          const float p = s[m] * kk[m];
+          if ((m & 3) == 0) d0 += p; else if ((m & 3) == 1) d1 += p; else if ((m & 3) == 2) d2 += p; else d3 += p;
         }
-        const float u = bt * (vc - row16_sum(d0 + d1));
+        const float u = bt * (vc - group_sum<RS>((d0 + d1) + (d2 + d3)));
 #pragma unroll
         for (int m = 0; m < KR; ++m) {
           s[m] += kk[m] * u;
-          if (m & 1) o1 += s[m] * qq[m]; else o0 += s[m] * qq[m];
+          const float p = s[m] * qq[m];
+          if ((m & 3) == 0) o0 += p; else if ((m & 3) == 1) o1 += p; else if ((m & 3) == 2) o2 += p; else o3 += p;
         }
       } else {
 #pragma unroll
         for (int m = 0; m < KR; ++m) {
-          s[m] = sa[tt][rg * KR + m] * s[m] + kk[m] * vc;
-          if (m & 1) o1 += s[m] * qq[m]; else o0 += s[m] * qq[m];
+          s[m] = sa[buf][tt][rg * KR + m] * s[m] + kk[m] * vc;
+          const float p = s[m] * qq[m];
+          if ((m & 3) == 0) o0 += p; else if ((m & 3) == 1) o1 += p; else if ((m & 3) == 2) o2 += p; else o3 += p;
         }
       }
-      const float o = row16_sum(o0 + o1);
+      const float o = group_sum<RS>((o0 + o1) + (o2 + o3));
       if (live && rg == 0) out[(int64_t)(t0 + tb + tt) * H * dv + h * dv + col] = o;
     }
+    if (more) stage(buf ^ 1);  // (its last readers passed the barrier that ended the previous block)
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
@@ -737,21 +824,21 @@ void gla_prep(const at::Tensor& P, int64_t a1_off, const at::Tensor& a2, const a
                                                          decay.data_ptr<float>());
 }
 
-template <bool DELTA>
+template <int RS, bool DELTA>
 void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* decay,
                 const float* beta, float q_scale, float* state, const int* slots, const int* cu, int H, int G, int d, int dv,
                 float* out) {
-#define REC_CASE(N)                                                                                                      \
-  case N:                                                                                                                \
-    linear_recurrence_k<N, DELTA><<<grid, 256, 0, stream()>>>(q, ldq, k, ldk, v, ldv, decay, beta, q_scale, state, slots, \
-                                                              cu, H, G, d, dv, out);                                     \
+#define REC_CASE(DPAD)                                                                                                 \
+  case DPAD:                                                                                                           \
+    linear_recurrence_k<DPAD / RS, RS, DELTA><<<grid, 256, 0, stream()>>>(q, ldq, k, ldk, v, ldv, decay, beta, q_scale, \
+                                                                          state, slots, cu, H, G, d, dv, out);         \
     break;
-  switch (KR) {
-    REC_CASE(1)
-    REC_CASE(2)
-    REC_CASE(4)
-    REC_CASE(8)
+  switch (KR * RS) {  // padded key dim
     REC_CASE(16)
+    REC_CASE(32)
+    REC_CASE(64)
+    REC_CASE(128)
+    REC_CASE(256)
     default:
       MCHECK(false, "linear_recurrence: key dim above 256");
   }
@@ -784,17 +871,27 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   } else {
     MCHECK(decay.numel() == T * H * d && G == H, "per-channel decay must be [T, H d] with one q / k head per value head");
   }
-  int KR = 1;
-  while (KR * 16 < d) KR *= 2;
-  const dim3 grid((unsigned)B, (unsigned)H, (unsigned)((dv + REC_COLS - 1) / REC_COLS));
-  if (delta)
-    launch_rec<true>(KR, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,
-                     decay.data_ptr<float>(), beta->data_ptr<float>(), (float)q_scale, state.data_ptr<float>(),
-                     state_slots.data_ptr<int>(), cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, out.data_ptr<float>());
-  else
-    launch_rec<false>(KR, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,
-                      decay.data_ptr<float>(), nullptr, (float)q_scale, state.data_ptr<float>(), state_slots.data_ptr<int>(),
-                      cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, out.data_ptr<float>());
+  int DP = 16;
+  while (DP < d) DP *= 2;
+  MCHECK(DP <= 256, "linear_recurrence: key dim above 256");
+  // row groups per value channel: 4 when (sequences x heads x channels) already give half the SIMDs a wave and a
+  // thread's rows stay within 16 registers, else 16 (measured at 8 x 2048 tokens, 16 heads: d 64 / dv 128 0.84 ms with
+  // 4 against 1.01 with 16; d 128 / dv 128 1.48 against 1.21)
+  const int64_t waves4 = B * H * ((dv + 63) / 64) * 4;
+  const int RS = (waves4 >= 512 && DP <= 64) ? 4 : 16;
+  const int cols = 256 / RS;
+  const dim3 grid((unsigned)B, (unsigned)H, (unsigned)((dv + cols - 1) / cols));
+  const float* bp = delta ? beta->data_ptr<float>() : nullptr;
+#define REC_GO(R, D)                                                                                                          \
+  launch_rec<R, D>(DP / R, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,              \
+                   decay.data_ptr<float>(), bp, (float)q_scale, state.data_ptr<float>(), state_slots.data_ptr<int>(),        \
+                   cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, out.data_ptr<float>())
+  if (RS == 4) {
+    if (delta) REC_GO(4, true); else REC_GO(4, false);
+  } else {
+    if (delta) REC_GO(16, true); else REC_GO(16, false);
+  }
+#undef REC_GO
 }
 
 void gated_rmsnorm(const at::Tensor& o, const at::Tensor& w, const at::Tensor& P, int64_t g_off, double eps, double out_scale,
