@@ -315,3 +315,32 @@ def test_greedy_generation_through_the_engine(dev):
     for t in range(len(p) - 1, len(seq) - 1):
       best = float(lg[t].max())
       assert float(lg[t][seq[t + 1]]) >= best - 0.05 * float(lg[t].std()), f"{rid}: token {t + 1} is not the greedy one"
+
+
+def test_checkpoint_directory_through_registry_and_engine(tmp_path):
+  """config.json + model.safetensors (bf16) in a folder: registered as a local model, loaded by the engine's own
+  build path, and the prompt's last-token logits match the oracle run on the same tensors."""
+  import json
+  from safetensors.torch import save_file
+  from xotorch_support_jetson_amd.download.shard_download import NoopShardDownloader
+  from xotorch_support_jetson_amd.inference.sharded_engine import ShardedInferenceEngine
+  from xotorch_support_jetson_amd.models import registry
+  cfg = SIZES[1]
+  c = from_hf_config(cfg)
+  tensors = random_mixed_tensors(c, 5)
+  (tmp_path / "config.json").write_text(json.dumps(cfg))
+  save_file({k: v.to(torch.bfloat16).contiguous() for k, v in tensors.items()}, str(tmp_path / "model.safetensors"))
+  mid = registry.register_local_model(str(tmp_path))
+  assert mid is not None and registry.model_cards[mid]["layers"] == len(cfg["layers"])
+  shard = registry.build_full_shard(mid, "ShardedInferenceEngine")
+  toks = [3, 99, 7, 7, 120, 64, 1, 0, 55]
+
+  async def main():
+    e = ShardedInferenceEngine(NoopShardDownloader(), device=torch.device("cpu"))
+    out, _ = await e.infer_tensor("r", shard, np.array([toks]), {})
+    return e, out
+  e, out = asyncio.run(main())
+  assert e.config.model_type == "tarepel" and e.config.layer_specs[1].rec.rank == 0 and e.runner.weights.layers[1].a2_w.shape[1] == 16
+  want = Oracle(cfg, tensors).logits(toks, want=[len(toks) - 1])[0]
+  got = out.double().reshape(-1)
+  assert (got - want).abs().max() < 0.03 * want.abs().max()  # bf16 activations on the serving path

@@ -67,7 +67,8 @@ def _batch(lens_done, lens_new, pages, dev, scramble):
 
 
 @pytest.mark.parametrize("dev,dtype", DEVS)
-@pytest.mark.parametrize("H,G,d,R,chunk", [(4, 2, 32, 16, 48), (2, 2, 64, 64, 64), (3, 1, 16, 0, 100), (2, 1, 128, 32, 7)])
+@pytest.mark.parametrize("H,G,d,R,chunk", [(4, 2, 32, 16, 48), (2, 2, 64, 64, 64), (3, 1, 16, 0, 100), (2, 1, 128, 32, 7),
+                                           (16, 1, 16, 8, 20), (6, 2, 20, 4, 33)])
 def test_chunked_sigmoid_attention(dev, dtype, H, G, d, R, chunk):
   D, scale, base = 24, 0.3, 1000.0
   lens = [150, 70]

@@ -215,6 +215,118 @@ __global__ void attn_gated_chunk_k(const AT* __restrict__ q, const AT* __restric
   }
 }
 
+// Single tokens and fp32 steps, query heads sharing a kv head (at most 8): workgroup = (token, kv head, key split).
+// Scores: a thread per key loads its K row once and scores it against every query head of the group.  Sum: threads
+// = value dims x key slices, 8 keys per 16-byte V^T load, one accumulator per query head; slices are reduced through
+// LDS.  With key splits each workgroup writes an fp32 partial and attn_split_sum_k adds them in a fixed order.
+constexpr int ATG_TILE = 256;
+constexpr int ATG_HEADS = 8;
+
+template <typename AT>
+__global__ __launch_bounds__(256) void attn_gated_chunk_gqa_k(
+    const AT* __restrict__ q, const AT* __restrict__ k_cache, const AT* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int B,
+    const float* __restrict__ pb, float scale, int chunk, float out_scale, AT* __restrict__ out, int ldo,
+    float* __restrict__ part, int T, int H, int G, int d, int dpad, int KS) {
+  extern __shared__ float sm[];
+  const int hpg = H / G;
+  float* qs = sm;                               // [hpg][d]
+  float* ws = qs + hpg * d;                     // [hpg][ATG_TILE + 8]
+  float* red = ws + hpg * (ATG_TILE + 8);       // [slices][hpg][dpad]
+  const int t = blockIdx.x, g = blockIdx.y, ks = blockIdx.z, tid = threadIdx.x;
+  const int b = seq_of(cu_q, B, t);
+  const int ctx = ctx_lens[b];
+  if (ctx <= 0) return;  // padding row of a captured decode batch
+  const int pos = ctx - (cu_q[b + 1] - cu_q[b]) + (t - cu_q[b]);
+  const int lo = (pos / chunk) * chunk;
+  // this split's keys [k0, k1): equal 8-aligned shares of [lo, pos]
+  const int share = (((pos - lo + 1) + KS - 1) / KS + 7) & ~7;
+  const int k0 = lo + ks * share, k1 = min(k0 + share, pos + 1);
+  for (int e = tid; e < hpg * d; e += 256) qs[e] = ldf(q + ((int64_t)t * H + g * hpg) * d + e);
+  const int nsl = 256 / dpad, di = tid % dpad, sl = tid / dpad;
+  const int* bt = block_tables + (int64_t)b * width;
+  float acc[ATG_HEADS];
+#pragma unroll
+  for (int hq = 0; hq < ATG_HEADS; ++hq) acc[hq] = 0.0f;
+  for (int p0 = k0; p0 < k1; p0 += ATG_TILE) {
+    const int p1 = min(p0 + ATG_TILE, k1);
+    const int a0 = p0 & ~7, a1 = (p1 + 7) & ~7;  // 8-aligned cover (<= ATG_TILE + 8 keys); outside [p0, p1) weighs 0
+    __syncthreads();
+    for (int p = a0 + tid; p < a1; p += 256) {
+      float sc[ATG_HEADS];
+#pragma unroll
+      for (int hq = 0; hq < ATG_HEADS; ++hq) sc[hq] = 0.0f;
+      const bool in = p >= p0 && p < p1;
+      if (in) {
+        const AT* kr = k_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * PAGE_TOK + (p % PAGE_TOK)) * d;
+        if (d & 7) {
+          for (int i = 0; i < d; ++i) {
+            const float kv = ldf(kr + i);
+#pragma unroll
+            for (int hq = 0; hq < ATG_HEADS; ++hq)
+              if (hq < hpg) sc[hq] += qs[hq * d + i] * kv;
+          }
+        } else {
+          for (int i = 0; i < d; i += 8) {
+            float kv[8];
+            ld8(kr + i, kv);
+#pragma unroll
+            for (int hq = 0; hq < ATG_HEADS; ++hq)
+              if (hq < hpg) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sc[hq] += qs[hq * d + i + e] * kv[e];
+              }
+          }
+        }
+      }
+#pragma unroll
+      for (int hq = 0; hq < ATG_HEADS; ++hq)
+        if (hq < hpg) ws[hq * (ATG_TILE + 8) + p - a0] = in ? sigmoidf_(sc[hq] * scale + pb[g * hpg + hq]) : 0.0f;
+    }
+    __syncthreads();
+    if (di < d) {
+      for (int p = a0 + 8 * sl; p < a1; p += 8 * nsl) {  // 8 keys of one page per step
+        float vv[8];
+        ld8(v_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * d + di) * PAGE_TOK + (p % PAGE_TOK), vv);
+#pragma unroll
+        for (int hq = 0; hq < ATG_HEADS; ++hq)
+          if (hq < hpg) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float w = ws[hq * (ATG_TILE + 8) + p - a0 + e];
+              acc[hq] += w != 0.0f ? w * vv[e] : 0.0f;  // (a slot no token has written yet may hold anything)
+            }
+          }
+      }
+    }
+  }
+#pragma unroll
+  for (int hq = 0; hq < ATG_HEADS; ++hq)
+    if (hq < hpg) red[(sl * hpg + hq) * dpad + di] = acc[hq];
+  __syncthreads();
+  for (int e = tid; e < hpg * d; e += 256) {
+    const int hq = e / d, i = e - hq * d;
+    float o = 0.0f;
+    for (int s2 = 0; s2 < nsl; ++s2) o += red[(s2 * hpg + hq) * dpad + i];
+    if (KS == 1)
+      stf(out + (int64_t)t * ldo + (g * hpg + hq) * d + i, o * out_scale);
+    else
+      part[((int64_t)ks * T + t) * H * d + (g * hpg + hq) * d + i] = o;
+  }
+}
+
+template <typename AT>
+__global__ void attn_split_sum_k(const float* __restrict__ part, int KS, int T, int HD, float out_scale, AT* __restrict__ out,
+                                 int ldo, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int B) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)T * HD) return;
+  const int t = (int)(idx / HD), i = (int)(idx - (int64_t)t * HD);
+  if (ctx_lens[seq_of(cu_q, B, t)] <= 0) return;  // padding row: no partials were written
+  float o = 0.0f;
+  for (int ks = 0; ks < KS; ++ks) o += part[((int64_t)ks * T + t) * HD + i];
+  stf(out + (int64_t)t * ldo + i, o * out_scale);
+}
+
 // MFMA kernel (bf16, d = 32 NK): a workgroup owns 128 consecutive queries of one (sequence, head), 32 per wave, and
 // walks the keys of their chunk(s) a tile of KT keys at a time: the K rows and V^T runs of the tile are staged in LDS
 // with whole-line loads and shared by the four waves.  Scores are computed transposed, S^T = K Q^T (keys x queries),
@@ -357,41 +469,45 @@ __global__ void delta_prep_k(const float* __restrict__ P, int ldp, int x_off, in
                              const int* __restrict__ state_slots, const int* __restrict__ cu_q, int B,
                              const float* __restrict__ A_log, const float* __restrict__ dt_bias, int H, int G, int d, int dv,
                              float* __restrict__ qkv, float* __restrict__ beta, float* __restrict__ decay) {
-  extern __shared__ float ys[];  // [C]
-  const int t = blockIdx.x;
+  // workgroup = (token, unit): units 0 .. G-1 the q heads, G .. 2G-1 the k heads, then H value heads, then the gates
+  __shared__ float red[16];
+  const int t = blockIdx.x, unit = blockIdx.y;
   const int b = seq_of(cu_q, B, t);
   const int slot = state_slots[b];
   if (slot < 0) return;
   const int C = 2 * G * d + H * dv;
-  const int local = t - cu_q[b];
+  if (unit == 2 * G + H) {
+    const float* row = P + (int64_t)t * ldp;
+    for (int h = threadIdx.x; h < H; h += blockDim.x) {
+      beta[(int64_t)t * H + h] = sigmoidf_(row[b_off + h]);
+      decay[(int64_t)t * H + h] = expf(-expf(A_log[h]) * softplusf_(row[a_off + h] + dt_bias[h]));
+    }
+    return;
+  }
+  const bool qk = unit < 2 * G;
+  const int c0 = qk ? unit * d : 2 * G * d + (unit - 2 * G) * dv, n = qk ? d : dv;
+  const int local = t - cu_q[b], tstart = cu_q[b];
   const float* st = conv_state + (int64_t)slot * (taps - 1) * C;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  float* o = qkv + (int64_t)t * C;
+  float ss = 0.0f;
+  // (n <= 256 in practice: one channel per thread; the loop keeps any size right)
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int c = c0 + i;
     float y = 0.0f;
     for (int j = 0; j < taps; ++j) {
-      const int s = local - (taps - 1 - j);
-      const float x = s >= 0 ? P[(int64_t)(cu_q[b] + s) * ldp + x_off + c] : st[(int64_t)(taps - 1 + s) * C + c];
+      const int sidx = local - (taps - 1 - j);
+      const float x = sidx >= 0 ? P[(int64_t)(tstart + sidx) * ldp + x_off + c] : st[(int64_t)(taps - 1 + sidx) * C + c];
       y += conv_w[c * taps + j] * x;
     }
-    ys[c] = siluf_(y);
+    y = siluf_(y);
+    o[c] = y;
+    ss += y * y;
   }
-  __syncthreads();
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
-  float* o = qkv + (int64_t)t * C;
-  for (int hd = wave; hd < 2 * G; hd += nw) {  // q heads then k heads
-    const float* y = ys + hd * d;
-    float ss = 0.0f;
-    for (int i = lane; i < d; i += 64) ss += y[i] * y[i];
-    ss = wave_sum(ss);
-    float k = 1.0f / sqrtf(ss + 1e-6f);
-    if (hd < G) k *= 1.0f / sqrtf((float)d);
-    for (int i = lane; i < d; i += 64) o[hd * d + i] = y[i] * k;
-  }
-  for (int c = 2 * G * d + threadIdx.x; c < C; c += blockDim.x) o[c] = ys[c];
-  for (int h = threadIdx.x; h < H; h += blockDim.x) {
-    const float* row = P + (int64_t)t * ldp;
-    beta[(int64_t)t * H + h] = sigmoidf_(row[b_off + h]);
-    decay[(int64_t)t * H + h] = expf(-expf(A_log[h]) * softplusf_(row[a_off + h] + dt_bias[h]));
-  }
+  if (!qk) return;
+  ss = block_sum(ss, red);
+  float kn = 1.0f / sqrtf(ss + 1e-6f);
+  if (unit < G) kn *= 1.0f / sqrtf((float)d);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) o[c0 + i] *= kn;  // each thread rescales what it wrote
 }
 
 __global__ void conv_state_update_k(const float* __restrict__ P, int ldp, int x_off, int C, int taps,
@@ -479,6 +595,49 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
 #pragma unroll
   for (int m = 0; m < KR; ++m) s[m] = (live && rg * KR + m < d) ? S[m] : 0.0f;
 
+  if (n == 1) {  // one decoded token: its k / q rows straight from memory, no staging and no barriers
+    float o0 = 0.0f, o1 = 0.0f, dd0 = 0.0f, dd1 = 0.0f;
+    const int64_t t = t0;
+    float kk[KR], qq[KR];
+#pragma unroll
+    for (int m = 0; m < KR; ++m) {
+      const int i = rg * KR + m;
+      const bool in = i < d;
+      kk[m] = in ? k[t * ldk + hk * d + i] : 0.0f;
+      qq[m] = in ? q[t * ldq + hk * d + i] * q_scale : 0.0f;
+    }
+    const float vc = live ? v[t * ldv + h * dv + col] : 0.0f;
+    if (DELTA) {
+      const float g = decay[t * H + h], bt = beta[t * H + h];
+#pragma unroll
+      for (int m = 0; m < KR; ++m) {
+        s[m] *= g;
+        if (m & 1) dd1 += s[m] * kk[m]; else dd0 += s[m] * kk[m];
+      }
+      const float u = bt * (vc - group_sum<RS>(dd0 + dd1));
+#pragma unroll
+      for (int m = 0; m < KR; ++m) {
+        s[m] += kk[m] * u;
+        if (m & 1) o1 += s[m] * qq[m]; else o0 += s[m] * qq[m];
+      }
+    } else {
+#pragma unroll
+      for (int m = 0; m < KR; ++m) {
+        const int i = rg * KR + m;
+        const float a = i < d ? decay[(t * H + h) * d + i] : 0.0f;
+        s[m] = a * s[m] + kk[m] * vc;
+        if (m & 1) o1 += s[m] * qq[m]; else o0 += s[m] * qq[m];
+      }
+    }
+    const float o = group_sum<RS>(o0 + o1);
+    if (live) {
+      if (rg == 0) out[t * H * dv + h * dv + col] = o;
+#pragma unroll
+      for (int m = 0; m < KR; ++m)
+        if (rg * KR + m < d) S[m] = s[m];
+    }
+    return;
+  }
   float pq[NQ], pk[NQ], pa[DELTA ? 1 : NQ], pv[NV], pg0 = 0.0f, pg1 = 0.0f;
   auto fetch = [&](int tb) {  // global -> registers: tokens tb .. tb + TB - 1 of the sequence (zeros past its end)
 #pragma unroll
@@ -755,6 +914,41 @@ void attn_gated_chunk(const at::Tensor& q, const at::Tensor& k_cache, const at::
 #undef ATT_CASE
     return;
   }
+  if (H / G <= ATG_HEADS) {
+    const int hpg = (int)(H / G);
+    int dpad = 16;
+    while (dpad < d) dpad *= 2;
+    // key splits: enough workgroups to cover the chip (about two per CU), at least 64 keys each
+    int KS = (int)std::min<int64_t>(std::min<int64_t>(8, (chunk + 63) / 64), (512 + T * G - 1) / (T * G));
+    KS = std::max(KS, 1);
+    at::Tensor part;
+    if (KS > 1) part = at::empty({KS, T, H * d}, q.options().dtype(at::kFloat));
+    const dim3 grid((unsigned)T, (unsigned)G, (unsigned)KS);
+    const size_t lds = ((size_t)hpg * d + (size_t)hpg * (ATG_TILE + 8) + (size_t)(256 / dpad) * hpg * dpad) * sizeof(float);
+    float* pp = KS > 1 ? part.data_ptr<float>() : nullptr;
+    const int blocks = (int)((T * H * d + 255) / 256);
+    if (bf) {
+      attn_gated_chunk_gqa_k<uint16_t><<<grid, 256, lds, stream()>>>(
+          (const uint16_t*)q.data_ptr(), (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(),
+          block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B,
+          pb.data_ptr<float>(), (float)scale, (int)chunk, (float)out_scale, (uint16_t*)out.data_ptr(), ldo, pp, (int)T, (int)H,
+          (int)G, (int)d, dpad, KS);
+      if (KS > 1)
+        attn_split_sum_k<uint16_t><<<blocks, 256, 0, stream()>>>(pp, KS, (int)T, (int)(H * d), (float)out_scale,
+                                                                 (uint16_t*)out.data_ptr(), ldo, cu_q.data_ptr<int>(),
+                                                                 ctx_lens.data_ptr<int>(), (int)B);
+    } else {
+      attn_gated_chunk_gqa_k<float><<<grid, 256, lds, stream()>>>(
+          q.data_ptr<float>(), k_cache.data_ptr<float>(), v_cache.data_ptr<float>(), block_tables.data_ptr<int>(),
+          (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, pb.data_ptr<float>(), (float)scale,
+          (int)chunk, (float)out_scale, out.data_ptr<float>(), ldo, pp, (int)T, (int)H, (int)G, (int)d, dpad, KS);
+      if (KS > 1)
+        attn_split_sum_k<float><<<blocks, 256, 0, stream()>>>(pp, KS, (int)T, (int)(H * d), (float)out_scale,
+                                                              out.data_ptr<float>(), ldo, cu_q.data_ptr<int>(),
+                                                              ctx_lens.data_ptr<int>(), (int)B);
+    }
+    return;
+  }
   const dim3 grid((unsigned)T, (unsigned)H);
   const size_t lds = (d + ATT_TILE + 8) * sizeof(float);
   if (bf)
@@ -794,8 +988,8 @@ void delta_prep(const at::Tensor& P, int64_t x_off, int64_t b_off, int64_t a_off
   cols_ok(P, x_off, C, "conv inputs");
   cols_ok(P, b_off, H, "beta");
   cols_ok(P, a_off, H, "decay");
-  MCHECK(C * sizeof(float) <= 64 * 1024, "delta_prep: too many convolution channels");
-  delta_prep_k<<<T, 256, C * sizeof(float), stream()>>>(
+  const int bs = std::min<int64_t>(256, ((std::max(d, dv) + 63) / 64) * 64);
+  delta_prep_k<<<dim3((unsigned)T, (unsigned)(2 * G + H + 1)), bs, 0, stream()>>>(
       P.data_ptr<float>(), ldp, (int)x_off, (int)b_off, (int)a_off, conv_w.data_ptr<float>(), (int)taps,
       conv_state.data_ptr<float>(), state_slots.data_ptr<int>(), cu_q.data_ptr<int>(), (int)B, A_log.data_ptr<float>(),
       dt_bias.data_ptr<float>(), (int)H, (int)G, (int)d, (int)dv, qkv.data_ptr<float>(), beta.data_ptr<float>(),
