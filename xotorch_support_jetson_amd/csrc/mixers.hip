@@ -592,52 +592,23 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
   const int hk = h / (H / G);
   float* S = state + (((int64_t)slot * H + h) * dv + (live ? col : 0)) * d + rg * KR;
   float s[KR];
+  // 16-byte state loads / stores where the thread's rows are whole float4s inside d (d and KR multiples of 4)
+  const bool vec = KR % 4 == 0 && (d & 3) == 0;
 #pragma unroll
-  for (int m = 0; m < KR; ++m) s[m] = (live && rg * KR + m < d) ? S[m] : 0.0f;
-
-  if (n == 1) {  // one decoded token: its k / q rows straight from memory, no staging and no barriers
-    float o0 = 0.0f, o1 = 0.0f, dd0 = 0.0f, dd1 = 0.0f;
-    const int64_t t = t0;
-    float kk[KR], qq[KR];
-#pragma unroll
-    for (int m = 0; m < KR; ++m) {
-      const int i = rg * KR + m;
-      const bool in = i < d;
-      kk[m] = in ? k[t * ldk + hk * d + i] : 0.0f;
-      qq[m] = in ? q[t * ldq + hk * d + i] * q_scale : 0.0f;
-    }
-    const float vc = live ? v[t * ldv + h * dv + col] : 0.0f;
-    if (DELTA) {
-      const float g = decay[t * H + h], bt = beta[t * H + h];
-#pragma unroll
-      for (int m = 0; m < KR; ++m) {
-        s[m] *= g;
-        if (m & 1) dd1 += s[m] * kk[m]; else dd0 += s[m] * kk[m];
-      }
-      const float u = bt * (vc - group_sum<RS>(dd0 + dd1));
-#pragma unroll
-      for (int m = 0; m < KR; ++m) {
-        s[m] += kk[m] * u;
-        if (m & 1) o1 += s[m] * qq[m]; else o0 += s[m] * qq[m];
-      }
+  for (int m = 0; m < KR; m += (KR % 4 == 0 ? 4 : 1)) {
+    if (KR % 4 == 0 && vec) {
+      const bool in = live && rg * KR + m + 4 <= d;
+      const f32x4 x = in ? *reinterpret_cast<const f32x4*>(S + m) : f32x4{0.f, 0.f, 0.f, 0.f};
+      s[m] = x[0];
+      s[m + 1] = x[1];
+      s[m + 2] = x[2];
+      s[m + 3] = x[3];
     } else {
 #pragma unroll
-      for (int m = 0; m < KR; ++m) {
-        const int i = rg * KR + m;
-        const float a = i < d ? decay[(t * H + h) * d + i] : 0.0f;
-        s[m] = a * s[m] + kk[m] * vc;
-        if (m & 1) o1 += s[m] * qq[m]; else o0 += s[m] * qq[m];
-      }
+      for (int e = 0; e < (KR % 4 == 0 ? 4 : 1); ++e) s[m + e] = (live && rg * KR + m + e < d) ? S[m + e] : 0.0f;
     }
-    const float o = group_sum<RS>(o0 + o1);
-    if (live) {
-      if (rg == 0) out[t * H * dv + h * dv + col] = o;
-#pragma unroll
-      for (int m = 0; m < KR; ++m)
-        if (rg * KR + m < d) S[m] = s[m];
-    }
-    return;
   }
+
   float pq[NQ], pk[NQ], pa[DELTA ? 1 : NQ], pv[NV], pg0 = 0.0f, pg1 = 0.0f;
   auto fetch = [&](int tb) {  // global -> registers: tokens tb .. tb + TB - 1 of the sequence (zeros past its end)
 #pragma unroll
@@ -727,8 +698,15 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
   }
   if (live) {
 #pragma unroll
-    for (int m = 0; m < KR; ++m)
-      if (rg * KR + m < d) S[m] = s[m];
+    for (int m = 0; m < KR; m += (KR % 4 == 0 ? 4 : 1)) {
+      if (KR % 4 == 0 && vec) {
+        if (rg * KR + m + 4 <= d) *reinterpret_cast<f32x4*>(S + m) = f32x4{s[m], s[m + 1], s[m + 2], s[m + 3]};
+      } else {
+#pragma unroll
+        for (int e = 0; e < (KR % 4 == 0 ? 4 : 1); ++e)
+          if (rg * KR + m + e < d) S[m + e] = s[m + e];
+      }
+    }
   }
 }
 
