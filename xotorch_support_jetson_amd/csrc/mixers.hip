@@ -378,19 +378,36 @@ __global__ __launch_bounds__(256) void attn_gated_chunk_mfma_k(
   const int* bt = block_tables + (int64_t)b * width;
   // sigmoid(s scale + bias) = 1 / (1 + 2^(s ea + eb))
   const float ea = -scale * 1.4426950408889634f, eb = -bias * 1.4426950408889634f;
-  for (int tb = t_lo; tb <= t_hi; tb += KT) {
+  // a thread's share of a tile: NCH 16-byte chunks of K and of V^T, fetched one tile ahead into registers
+  constexpr int NCHUNK = KT * (D / 8), NCH = (NCHUNK + 255) / 256;
+  s16x8 rk[NCH], rv[NCH];
+  auto fetch = [&](int tb) {
     const int64_t pg = (int64_t)bt[tb >> 6] * G + gk;
     const int koff = tb & 63;
-    __syncthreads();  // the previous tile has been consumed
-    for (int ch = threadIdx.x; ch < KT * (D / 8); ch += 256) {
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int ch = threadIdx.x + 256 * j;
+      if (NCHUNK % 256 != 0 && ch >= NCHUNK) break;
       const int row = ch / (D / 8), cc = ch - row * (D / 8);
-      st16(&sK[row][cc * 8], ld16(k_cache + ((pg * PAGE_TOK) + koff + row) * D + cc * 8));
+      rk[j] = ld16(k_cache + ((pg * PAGE_TOK) + koff + row) * D + cc * 8);
+      const int vrow = ch / (KT / 8), vc = ch - vrow * (KT / 8);
+      rv[j] = ld16(v_cache + (pg * D + vrow) * PAGE_TOK + koff + vc * 8);
     }
-    for (int ch = threadIdx.x; ch < D * (KT / 8); ch += 256) {
-      const int row = ch / (KT / 8), cc = ch - row * (KT / 8);
-      st16(&sV[row][cc * 8], ld16(v_cache + (pg * D + row) * PAGE_TOK + koff + cc * 8));
+  };
+  fetch(t_lo);
+  for (int tb = t_lo; tb <= t_hi; tb += KT) {
+    __syncthreads();  // the previous tile has been consumed
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int ch = threadIdx.x + 256 * j;
+      if (NCHUNK % 256 != 0 && ch >= NCHUNK) break;
+      const int row = ch / (D / 8), cc = ch - row * (D / 8);
+      st16(&sK[row][cc * 8], rk[j]);
+      const int vrow = ch / (KT / 8), vc = ch - vrow * (KT / 8);
+      st16(&sV[vrow][vc * 8], rv[j]);
     }
     __syncthreads();
+    if (tb + KT <= t_hi) fetch(tb + KT);  // in flight while this tile is consumed
 #pragma unroll
     for (int sub = 0; sub < KT / 32; ++sub) {
       const int kb = tb + sub * 32;
