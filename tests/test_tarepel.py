@@ -203,7 +203,7 @@ SIZES = [
   # one head everywhere, kv_heads == heads, full rotation, chunk of one page, two taps
   config([par(attn(1, 1, 32, 64, 32), delta(1, 1, 32, 32, 2)), gla(1, 16, 16, 1.0)], width=48, vocab=50, logit_scale=1.0),
   # rotation on a quarter of the head, chunk shorter than a page and not dividing it, wide heads, five taps
-  config([par(attn(6, 3, 128, 40, 32, 1e6, 0.09), delta(6, 3, 64, 64, 5), ff=160, ls=1.3, rs=0.4), gla(3, 64, 128, 16.0)],
+  config([par(attn(6, 3, 128, 40, 32, 1e6, 0.09), delta(6, 2, 64, 48, 5), ff=160, ls=1.3, rs=0.4), gla(3, 64, 128, 16.0)],
          width=160, vocab=130),
   # chunk longer than a page, no rotation at all, key dim above value dim, a layer without feed-forward first
   config([gla(2, 48, 16, 2.0, ff=0), par(attn(2, 1, 16, 100, 0), delta(3, 3, 48, 16, 4), ff=32)], width=32, vocab=40),
@@ -340,7 +340,7 @@ def test_checkpoint_directory_through_registry_and_engine(tmp_path):
     out, _ = await e.infer_tensor("r", shard, np.array([toks]), {})
     return e, out
   e, out = asyncio.run(main())
-  assert e.config.model_type == "tarepel" and e.config.layer_specs[1].rec.rank == 0 and e.runner.weights.layers[1].a2_w.shape[1] == 16
+  assert e.config.model_type == "tarepel" and e.config.layer_specs[1].rec.rank == 0 and e.runner.weights.layers[1].a2_w.shape[1] == 8
   want = Oracle(cfg, tensors).logits(toks, want=[len(toks) - 1])[0]
   got = out.double().reshape(-1)
   assert (got - want).abs().max() < 0.03 * want.abs().max()  # bf16 activations on the serving path

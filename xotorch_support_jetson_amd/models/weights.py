@@ -772,7 +772,7 @@ def mixed_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
       out[m + "b"], out[m + "a"], out[m + "A_log"], out[m + "dt_bias"] = (r.heads, D), (r.heads, D), (r.heads,), (r.heads,)
       out[m + "norm"], out[m + "g"], out[m + "o"] = (r.vdim,), (r.heads * r.vdim, D), (D, r.heads * r.vdim)
     elif r is not None:
-      m, rank = p + "mix.", r.rank or 16
+      m, rank = p + "mix.", r.rank or 8
       out[m + "q"], out[m + "k"], out[m + "v"] = (r.heads * r.dim, D), (r.heads * r.dim, D), (r.heads * r.vdim, D)
       out[m + "g"], out[m + "o"], out[m + "norm"] = (r.heads * r.vdim, D), (D, r.heads * r.vdim), (r.vdim,)
       out[m + "a1"], out[m + "a2"], out[m + "a2.b"] = (rank, D), (r.heads * r.dim, rank), (r.heads * r.dim,)
