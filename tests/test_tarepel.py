@@ -344,3 +344,55 @@ def test_checkpoint_directory_through_registry_and_engine(tmp_path):
   want = Oracle(cfg, tensors).logits(toks, want=[len(toks) - 1])[0]
   got = out.double().reshape(-1)
   assert (got - want).abs().max() < 0.03 * want.abs().max()  # bf16 activations on the serving path
+
+
+@pytest.mark.parametrize("dev,dtype", RUNS)
+def test_two_pipeline_shards_match_one(dev, dtype):
+  """Layers 0-1 on one runner, 2-3 on another (the fp32 residual stream travels between them): the same logits as
+  the unsplit model, in portions and token by token."""
+  c = from_hf_config(SMALL)
+  tensors = random_mixed_tensors(c, 11)
+  n = c.num_layers
+  runners = []
+  for lo, hi in ((0, 1), (2, n - 1)):
+    shard = Shard("t", lo, hi, n)
+    w = mixed_weights(c, shard, tensors.__getitem__, torch.device(dev), dtype)
+    runners.append(ShardRunner(c, shard, torch.device(dev), weights=w, num_pages=8, max_batch=2, max_ctx=512, dtype=dtype))
+  assert runners[0].hidden_dtype == torch.float32
+  toks = torch.randint(0, c.vocab_size, (90,), generator=torch.Generator().manual_seed(3)).tolist()
+  outs, lo = [], 0
+  for m in (40, 1, 1, 30, 2, 16):
+    ids = torch.tensor(toks[lo:lo + m], dtype=torch.int32)
+    hidden = runners[0].forward(["a"], [m], ids)
+    assert hidden.dtype == torch.float32 and tuple(hidden.shape) == (m, c.hidden_size)
+    outs.append(runners[1].forward(["a"], [m], hidden.clone(), logit_rows=list(range(m))).double().cpu())
+    lo += m
+  want = Oracle(SMALL, tensors).logits(toks)
+  d = torch.cat(outs) - want
+  d = d - d.mean(-1, keepdim=True)
+  assert (d.pow(2).mean(-1).sqrt() / want.pow(2).mean().sqrt()).max() < TOL[dtype]
+
+
+def test_native_slot_manager_matches_python_twin():
+  _runtime = pytest.importorskip("xotorch_support_jetson_amd._runtime")
+  from xotorch_support_jetson_amd.runtime.runner import SlotManager
+  a, b = _runtime.SlotManager(3), SlotManager(3)
+  g = torch.Generator().manual_seed(0)
+  live = []
+  for step in range(200):
+    if live and (len(live) == 3 or int(torch.randint(0, 2, (1,), generator=g))):
+      rid = live.pop(int(torch.randint(0, len(live), (1,), generator=g)))
+      a.release(rid)
+      b.release(rid)
+    else:
+      rid = f"r{step}"
+      assert a.acquire(rid) == b.acquire(rid)
+      live.append(rid)
+    assert a.num_free == b.num_free and all(a.slot(r) == b.slot(r) and a.has(r) for r in live)
+  for m in (a, b):
+    for r in list(live):
+      m.release(r)
+    for i in range(3):
+      assert m.acquire(f"x{i}") == i
+    with pytest.raises(RuntimeError, match="state slots"):
+      m.acquire("y")

@@ -4,6 +4,7 @@
 #include <pybind11/stl.h>
 
 #include "block_manager.h"
+#include "slot_manager.h"
 
 namespace py = pybind11;
 
@@ -36,4 +37,12 @@ PYBIND11_MODULE(_runtime, m) {
       .def("block_table", &xot_rt::BlockManager::block_table)
       .def("fill_batch", &fill_batch_np)
       .def("check", &xot_rt::BlockManager::check);
+  py::class_<xot_rt::SlotManager>(m, "SlotManager")
+      .def(py::init<int64_t>(), py::arg("slots"))
+      .def_property_readonly("slots", &xot_rt::SlotManager::slots)
+      .def_property_readonly("num_free", &xot_rt::SlotManager::num_free)
+      .def("has", &xot_rt::SlotManager::has)
+      .def("slot", &xot_rt::SlotManager::slot)
+      .def("acquire", &xot_rt::SlotManager::acquire)
+      .def("release", &xot_rt::SlotManager::release);
 }

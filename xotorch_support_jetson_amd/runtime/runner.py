@@ -31,9 +31,18 @@ def _block_manager(num_pages: int):
     return BlockManager(num_pages, PAGE)
 
 
+def _slot_manager(slots: int):
+  try:
+    from .. import _runtime
+    return _runtime.SlotManager(slots)
+  except (ImportError, AttributeError):
+    return SlotManager(slots)  # pure-python twin for hosts without the build
+
+
 class SlotManager:
   """State slots of models with recurrent layers: one slot per live request, handed out on admission and returned
-  when the request ends (lowest free slot first, so a small pool is reused at once)."""
+  when the request ends (lowest free slot first, so a small pool is reused at once).  Python twin of the native
+  class (csrc/runtime/slot_manager.h), used where the C++ runtime is not built and as its executable specification."""
 
   def __init__(self, slots: int):
     self.slots = slots
@@ -51,6 +60,8 @@ class SlotManager:
     return self._of[rid]
 
   def acquire(self, rid: str) -> int:
+    if rid in self._of:
+      raise ValueError(f"request {rid} already holds a state slot")
     if not self._free:
       raise RuntimeError(f"state slots exhausted: all {self.slots} are held by live requests")
     s = self._of[rid] = self._free.pop()
@@ -114,7 +125,7 @@ class ShardRunner:
       KVCache(config, n_layers, num_pages, self.device)
     self.bm = _block_manager(num_pages)
     # recurrent layers: one state slot per live request (max_batch of them), cleared on admission
-    self.sm = SlotManager(max_batch) if config.has_state else None
+    self.sm = _slot_manager(max_batch) if config.has_state else None
     self.state = StatePool(config, shard.layers(), max_batch, self.device) if config.has_state else None
     self.max_ctx = max_ctx
     self.max_batch = max_batch
