@@ -485,17 +485,20 @@ __global__ void delta_prep_k(const float* __restrict__ P, int ldp, int x_off, in
                              const float* __restrict__ conv_w, int taps, const float* __restrict__ conv_state,
                              const int* __restrict__ state_slots, const int* __restrict__ cu_q, int B,
                              const float* __restrict__ A_log, const float* __restrict__ dt_bias, int H, int G, int d, int dv,
-                             float* __restrict__ qkv, float* __restrict__ beta, float* __restrict__ decay) {
-  // workgroup = (token, unit): units 0 .. G-1 the q heads, G .. 2G-1 the k heads, then H value heads, then the gates
-  __shared__ float red[16];
-  const int t = blockIdx.x, unit = blockIdx.y;
-  const int b = seq_of(cu_q, B, t);
-  const int slot = state_slots[b];
-  if (slot < 0) return;
+                             float* __restrict__ qkv, float* __restrict__ beta, float* __restrict__ decay, int T, int tpb) {
+  // workgroup = (tpb <= 8 consecutive tokens, unit): units 0 .. G-1 the q heads, G .. 2G-1 the k heads, then H value
+  // heads, then the gates.  A thread owns one channel of the unit for all the tokens: their convolution inputs are
+  // loaded together and the tokens' sums of squares are reduced in one pass.  tpb is 1 for decode steps.
+  constexpr int TPB = 8;
+  __shared__ float red[TPB][4];
+  const int unit = blockIdx.y;
   const int C = 2 * G * d + H * dv;
+  const int tbase = blockIdx.x * tpb;
   if (unit == 2 * G + H) {
-    const float* row = P + (int64_t)t * ldp;
-    for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    for (int e = threadIdx.x; e < tpb * H; e += blockDim.x) {
+      const int t = tbase + e / H, h = e % H;
+      if (t >= T || state_slots[seq_of(cu_q, B, t)] < 0) continue;
+      const float* row = P + (int64_t)t * ldp;
       beta[(int64_t)t * H + h] = sigmoidf_(row[b_off + h]);
       decay[(int64_t)t * H + h] = expf(-expf(A_log[h]) * softplusf_(row[a_off + h] + dt_bias[h]));
     }
@@ -503,28 +506,53 @@ __global__ void delta_prep_k(const float* __restrict__ P, int ldp, int x_off, in
   }
   const bool qk = unit < 2 * G;
   const int c0 = qk ? unit * d : 2 * G * d + (unit - 2 * G) * dv, n = qk ? d : dv;
-  const int local = t - cu_q[b], tstart = cu_q[b];
-  const float* st = conv_state + (int64_t)slot * (taps - 1) * C;
-  float* o = qkv + (int64_t)t * C;
-  float ss = 0.0f;
-  // (n <= 256 in practice: one channel per thread; the loop keeps any size right)
-  for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    const int c = c0 + i;
-    float y = 0.0f;
+  const int i = threadIdx.x;  // the launch gives a thread per channel of the widest unit (n <= blockDim.x <= 256)
+  const int c = c0 + i;
+  float y[TPB];
+  bool ok[TPB];
+#pragma unroll
+  for (int tt = 0; tt < TPB; ++tt) {
+    const int t = tbase + tt;
+    y[tt] = 0.0f;
+    ok[tt] = false;
+    if (tt >= tpb || t >= T) continue;
+    const int b = seq_of(cu_q, B, t);
+    const int slot = state_slots[b];
+    if (slot < 0) continue;
+    ok[tt] = true;
+    if (i >= n) continue;
+    const int local = t - cu_q[b], tstart = cu_q[b];
+    const float* st = conv_state + (int64_t)slot * (taps - 1) * C;
+    float acc = 0.0f;
     for (int j = 0; j < taps; ++j) {
       const int sidx = local - (taps - 1 - j);
       const float x = sidx >= 0 ? P[(int64_t)(tstart + sidx) * ldp + x_off + c] : st[(int64_t)(taps - 1 + sidx) * C + c];
-      y += conv_w[c * taps + j] * x;
+      acc += conv_w[c * taps + j] * x;
     }
-    y = siluf_(y);
-    o[c] = y;
-    ss += y * y;
+    y[tt] = siluf_(acc);
   }
-  if (!qk) return;
-  ss = block_sum(ss, red);
-  float kn = 1.0f / sqrtf(ss + 1e-6f);
-  if (unit < G) kn *= 1.0f / sqrtf((float)d);
-  for (int i = threadIdx.x; i < n; i += blockDim.x) o[c0 + i] *= kn;  // each thread rescales what it wrote
+  if (qk) {
+    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+#pragma unroll
+    for (int tt = 0; tt < TPB; ++tt) {
+      const float ss = wave_sum(y[tt] * y[tt]);
+      if ((threadIdx.x & 63) == 0) red[tt][wave] = ss;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < TPB; ++tt) {
+      float ss = 0.0f;
+      for (int w = 0; w < nw; ++w) ss += red[tt][w];
+      float kn = 1.0f / sqrtf(ss + 1e-6f);
+      if (unit < G) kn *= 1.0f / sqrtf((float)d);
+      y[tt] *= kn;
+    }
+  }
+  if (i < n) {
+#pragma unroll
+    for (int tt = 0; tt < TPB; ++tt)
+      if (ok[tt]) qkv[(int64_t)(tbase + tt) * C + c] = y[tt];
+  }
 }
 
 __global__ void conv_state_update_k(const float* __restrict__ P, int ldp, int x_off, int C, int taps,
@@ -565,9 +593,8 @@ __global__ void gla_prep_k(const float* __restrict__ P, int ldp, int a1_off, int
 // Workgroup = (sequence, value head, 256 / RS value channels); 256 threads = channels x RS row groups, the row group
 // in the low lane bits: the two dot products reduce inside DPP rows, register to register.  A thread keeps the KR
 // consecutive key rows rg KR .. rg KR + KR - 1 of its channel in registers (d <= RS KR), so state loads and stores are
-// contiguous runs and a token's k / q slices are vector LDS reads.  RS = 4 does the least work per state element (the
-// choice when sequences x heads x channels fill the chip); RS = 16 spreads one (sequence, head) over four times the
-// lanes.  Tokens are staged through LDS TB at a time, double-buffered: the next block's global loads are in flight
+// contiguous runs and a token's k / q slices are vector LDS reads.  The launcher uses RS = 16 (a whole DPP row per
+// value channel).  Tokens are staged through LDS TB at a time, double-buffered: the next block's global loads are in flight
 // while the current one is consumed.
 // DELTA: S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q.   else: S = diag(a) S + k v^T; o = S^T q.
 template <int CTRL>
@@ -581,10 +608,8 @@ template <int RS>
 __device__ __forceinline__ float group_sum(float v) {
   v = dpp_add<0xB1>(v);  // quad_perm [1, 0, 3, 2]
   v = dpp_add<0x4E>(v);  // quad_perm [2, 3, 0, 1]
-  if (RS == 16) {
-    v = dpp_add<0x141>(v);  // row_half_mirror
-    v = dpp_add<0x140>(v);  // row_mirror
-  }
+  if (RS >= 8) v = dpp_add<0x141>(v);   // row_half_mirror
+  if (RS == 16) v = dpp_add<0x140>(v);  // row_mirror
   return v;
 }
 
@@ -983,12 +1008,14 @@ void delta_prep(const at::Tensor& P, int64_t x_off, int64_t b_off, int64_t a_off
   cols_ok(P, x_off, C, "conv inputs");
   cols_ok(P, b_off, H, "beta");
   cols_ok(P, a_off, H, "decay");
-  const int bs = std::min<int64_t>(256, ((std::max(d, dv) + 63) / 64) * 64);
-  delta_prep_k<<<dim3((unsigned)T, (unsigned)(2 * G + H + 1)), bs, 0, stream()>>>(
+  MCHECK(d <= 256 && dv <= 256, "delta_prep: head sizes above 256");
+  const int bs = (int)(((std::max(d, dv) + 63) / 64) * 64);
+  const int tpb = T > 256 ? 8 : 1;
+  delta_prep_k<<<dim3((unsigned)((T + tpb - 1) / tpb), (unsigned)(2 * G + H + 1)), bs, 0, stream()>>>(
       P.data_ptr<float>(), ldp, (int)x_off, (int)b_off, (int)a_off, conv_w.data_ptr<float>(), (int)taps,
       conv_state.data_ptr<float>(), state_slots.data_ptr<int>(), cu_q.data_ptr<int>(), (int)B, A_log.data_ptr<float>(),
       dt_bias.data_ptr<float>(), (int)H, (int)G, (int)d, (int)dv, qkv.data_ptr<float>(), beta.data_ptr<float>(),
-      decay.data_ptr<float>());
+      decay.data_ptr<float>(), (int)T, tpb);
   if (taps > 1) {
     const dim3 grid((unsigned)B, (unsigned)((C + 255) / 256));
     conv_state_update_k<<<grid, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)x_off, (int)C, (int)taps,
@@ -1063,11 +1090,9 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   int DP = 16;
   while (DP < d) DP *= 2;
   MCHECK(DP <= 256, "linear_recurrence: key dim above 256");
-  // row groups per value channel: 4 when (sequences x heads x channels) already give half the SIMDs a wave and a
-  // thread's rows stay within 16 registers, else 16 (measured at 8 x 2048 tokens, 16 heads: d 64 / dv 128 0.84 ms with
-  // 4 against 1.01 with 16; d 128 / dv 128 1.48 against 1.21)
-  const int64_t waves4 = B * H * ((dv + 63) / 64) * 4;
-  const int RS = (waves4 >= 512 && DP <= 64) ? 4 : 16;
+  // 16 row groups per value channel (4 and 8, with more rows per thread, measured slower at 8 x 2048 tokens and 16
+  // heads: d 64 / dv 128 0.89 / 0.75 / 0.70 ms with 4 / 8 / 16, d 128 / dv 128 1.57 / 1.28 / 1.23)
+  const int RS = 16;
   const int cols = 256 / RS;
   const dim3 grid((unsigned)B, (unsigned)H, (unsigned)((dv + cols - 1) / cols));
   const float* bp = delta ? beta->data_ptr<float>() : nullptr;
@@ -1075,11 +1100,7 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   launch_rec<R, D>(DP / R, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,              \
                    decay.data_ptr<float>(), bp, (float)q_scale, state.data_ptr<float>(), state_slots.data_ptr<int>(),        \
                    cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, out.data_ptr<float>())
-  if (RS == 4) {
-    if (delta) REC_GO(4, true); else REC_GO(4, false);
-  } else {
-    if (delta) REC_GO(16, true); else REC_GO(16, false);
-  }
+  if (delta) REC_GO(16, true); else REC_GO(16, false);
 #undef REC_GO
 }
 
