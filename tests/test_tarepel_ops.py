@@ -68,7 +68,8 @@ def _batch(lens_done, lens_new, pages, dev, scramble):
 
 @pytest.mark.parametrize("dev,dtype", DEVS)
 @pytest.mark.parametrize("H,G,d,R,chunk", [(4, 2, 32, 16, 48), (2, 2, 64, 64, 64), (3, 1, 16, 0, 100), (2, 1, 128, 32, 7),
-                                           (16, 1, 16, 8, 20), (6, 2, 20, 4, 33)])
+                                           (16, 1, 16, 8, 20), (6, 2, 20, 4, 33), (2, 1, 96, 32, 50), (4, 2, 160, 160, 64),
+                                           (2, 2, 256, 64, 70), (2, 1, 224, 2, 130)])
 def test_chunked_sigmoid_attention(dev, dtype, H, G, d, R, chunk):
   D, scale, base = 24, 0.3, 1000.0
   lens = [150, 70]
@@ -121,7 +122,8 @@ def _slots_batch(lens_new, slots, dev):
 
 
 @pytest.mark.parametrize("dev,dtype", DEVS)
-@pytest.mark.parametrize("H,G,d,dv,taps", [(4, 2, 16, 32, 3), (2, 2, 64, 64, 4), (3, 1, 24, 80, 2), (1, 1, 128, 16, 5)])
+@pytest.mark.parametrize("H,G,d,dv,taps", [(4, 2, 16, 32, 3), (2, 2, 64, 64, 4), (3, 1, 24, 80, 2), (1, 1, 128, 16, 5),
+                                           (2, 1, 256, 40, 1), (2, 2, 200, 256, 3)])
 def test_gated_delta_rule(dev, dtype, H, G, d, dv, taps):
   D, eps = 20, 1e-5
   lens = [45, 9]
@@ -165,7 +167,8 @@ def test_gated_delta_rule(dev, dtype, H, G, d, dv, taps):
 
 
 @pytest.mark.parametrize("dev,dtype", DEVS)
-@pytest.mark.parametrize("H,d,dv,rank,tau", [(2, 32, 64, 8, 8.0), (4, 16, 16, 4, 1.0), (1, 100, 72, 16, 16.0), (3, 64, 130, 5, 3.0)])
+@pytest.mark.parametrize("H,d,dv,rank,tau", [(2, 32, 64, 8, 8.0), (4, 16, 16, 4, 1.0), (1, 100, 72, 16, 16.0), (3, 64, 130, 5, 3.0),
+                                             (2, 256, 48, 3, 2.0), (1, 8, 8, 1, 4.0)])
 def test_gated_linear_attention(dev, dtype, H, d, dv, rank, tau):
   D, eps = 20, 1e-5
   lens = [60, 33]
@@ -198,3 +201,46 @@ def test_gated_linear_attention(dev, dtype, H, d, dv, rank, tau):
       done[i] += new[i]
   for i in range(2):
     close(torch.cat(got[i]), want[i], dtype, f"gated linear attention, sequence {i}")
+
+
+@pytest.mark.parametrize("dev,dtype", DEVS)
+@pytest.mark.parametrize("chunk,d", [(48, 32), (64, 64), (100, 32), (32, 128), (7, 32)])
+def test_chunk_mask_is_exact(dev, dtype, chunk, d):
+  """Queries and a few marked keys point along one unrotated dim, with a bias of -12: a marked key weighs 0.98, every
+  other key 6e-6.  The marked keys sit on both sides of every chunk edge (and at position 0), so a key let in from
+  the previous chunk, a key of the own chunk left out, or a future key changes the output by its whole value.
+  Prompt portions (the MFMA kernel in bf16) and single decoded tokens."""
+  H, G, R, n = 2, 1, 16, 230
+  hq, hk = H * d, G * d
+  W = {"q": torch.cat([torch.eye(hq, dtype=torch.float64), torch.zeros(hq, hk, dtype=torch.float64)], 1),
+       "k": torch.cat([torch.zeros(hk, hq, dtype=torch.float64), torch.eye(hk, dtype=torch.float64)], 1),
+       "pb": torch.full((H,), -12.0, dtype=torch.float64), "o": torch.eye(hq, dtype=torch.float64)}
+  m = {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "mask": {"size": chunk}, "rot": {"dims": R, "base": 100.0}, "scale": 1.0}
+  marked = {0} | {c + o for c in range(chunk, n, chunk) for o in (-1, 0)} | {n - 1}
+  q = torch.zeros(n, H, d, dtype=torch.float64)
+  q[:, :, d - 1] = 4.0
+  k = 0.01 * rnd(n, G, d, seed=3)
+  for p in marked:
+    k[p, :, d - 1] = 4.0
+    k[p, :, 0] = 1.0 + p  # tells the marked keys apart in the output (rotated dim: only the value keeps it as is)
+  hs = torch.cat([q.reshape(n, -1), k.reshape(n, -1)], 1)
+  mem = {}
+  want = torch.stack([O.chunk_gated_attention(W, "", m, hs[p], p, mem) for p in range(n)])
+  from xotorch_support_jetson_amd.ops.rope import build_cos_sin
+  tab = build_cos_sin(R, 256, 100.0, None, dev)
+  kc = torch.zeros(4, G, 64, d, dtype=dtype, device=dev)
+  vc = torch.zeros(4, G, d, 64, dtype=dtype, device=dev)
+  got, done = [], 0
+  for new in [101, 2, 60] + [1] * (n - 163):
+    tables, slots, pos, cu, ctx = _batch([done], [new], 4, dev, scramble=9)
+    P = hs[done:done + new].float().to(dev)
+    qo = torch.empty(new, H, d, dtype=dtype, device=dev)
+    K.rope_kv_store(P, 0, hq, -1, H, G, d, R, pos, tab, slots, qo, kc, vc)
+    out = torch.zeros(new, hq, dtype=dtype, device=dev)
+    K.attn_gated_chunk(qo, kc, vc, tables, cu, ctx, W["pb"].float().to(dev), 1.0, chunk, 1.0, out, max_qlen=new)
+    got.append(out)
+    done += new
+  got = torch.cat(got).double().cpu()
+  err = (got - want).abs().max(-1).values / want.abs().max()
+  tol = 1e-4 if dtype == torch.float32 else 2e-2
+  assert err.max() < tol, f"position {int(err.argmax())} (chunk {chunk}) is off by {float(err.max()):.3g}"
