@@ -72,7 +72,9 @@ class RingStage:
     self.vs = int(V * frac) // 256 * 256
     want = os.environ.get("XOT_SPLIT_HEAD", "1") == "1" if split_head is None else split_head
     # the decision depends only on config and arguments, so every rank takes the same one
-    self.split = bool(want and world > 1 and 0 < self.vs < V and 1 <= top_k <= KC and top_k < self.vs)
+    # (mixed-layer models keep their scaled head whole on the last stage)
+    self.split = bool(want and world > 1 and 0 < self.vs < V and 1 <= top_k <= KC and top_k < self.vs
+                      and not runner.config.is_mixed)
     self.head_tail = None
     if self.split and self.first:
       self.head_tail = runner.head_tail(self.vs)
@@ -172,7 +174,7 @@ class RingStage:
         meta = torch.empty(1, dtype=torch.int64, device=dev)
         self.t.recv(meta, self.prev)
         Lc = int(meta.item())
-        x = torch.empty(n * Lc, self.D, dtype=torch.bfloat16, device=dev)
+        x = torch.empty(n * Lc, self.D, dtype=self.r.hidden_dtype, device=dev)
         self.t.recv(x, self.prev)
       y = self.r.forward(rids, [Lc] * n, x)
       if not self.last:
@@ -210,7 +212,7 @@ class RingStage:
         self.t.wait(self.t.irecv(x, self.prev))
         e1 = self._mark()
     else:
-      x = torch.empty(B, self.D, dtype=torch.bfloat16, device=dev)
+      x = torch.empty(B, self.D, dtype=self.r.hidden_dtype, device=dev)
       self.t.wait(self.t.irecv(x, self.prev))
       e1 = self._mark()
     y = self.r.forward(mb.rids, [1] * B, x)

@@ -316,7 +316,7 @@ class RingServer:
         at, prev, rows = gather
         x.index_copy_(0, at, prev.index_select(0, rows))
     else:
-      x = torch.empty(sum(qlens), self.D, dtype=torch.bfloat16, device=self.dev)
+      x = torch.empty(sum(qlens), self.D, dtype=self.r.hidden_dtype, device=self.dev)
       self.t.wait(self.t.irecv(x, self.prev))
     y = (self.r.forward(rids, qlens, x) if image_embeds is None
          else self.r.forward(rids, qlens, x, image_embeds=image_embeds))
