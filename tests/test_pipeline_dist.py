@@ -20,13 +20,13 @@ MODEL = "tiny-llama"
 B, L, STEPS = 3, 10, 5
 
 
-def _prompts(m):
+def _prompts(m, model=MODEL):
   g = torch.Generator().manual_seed(100 + m)
-  return torch.randint(0, PRESETS[MODEL].vocab_size, (B, L), generator=g, dtype=torch.int32)
+  return torch.randint(0, PRESETS[model].vocab_size, (B, L), generator=g, dtype=torch.int32)
 
 
-def _run(stage, n_mb):
-  mbs = [MicroBatch([f"m{m}r{b}" for b in range(B)], prompt=_prompts(m), temps=torch.zeros(B)) for m in range(n_mb)]
+def _run(stage, n_mb, model=MODEL):
+  mbs = [MicroBatch([f"m{m}r{b}" for b in range(B)], prompt=_prompts(m, model), temps=torch.zeros(B)) for m in range(n_mb)]
   first = [stage.prefill(mb) for mb in mbs]
   for mb, t in zip(mbs, first):
     if t is not None and not stage.split:  # split head: the prefill token is drawn by the first stage
@@ -35,16 +35,16 @@ def _run(stage, n_mb):
   return [mb.tokens for mb in mbs]
 
 
-def _worker(rank, world, port, q, split):
+def _worker(rank, world, port, q, split, model=MODEL):
   os.environ.update(MASTER_ADDR="127.0.0.1", MASTER_PORT=str(port), RANK=str(rank), WORLD_SIZE=str(world))
   dist.init_process_group("gloo", rank=rank, world_size=world)
   try:
-    c = PRESETS[MODEL]
-    shard = equal_layer_shards(MODEL, c.num_layers, world)[rank]
+    c = PRESETS[model]
+    shard = equal_layer_shards(model, c.num_layers, world)[rank]
     runner = ShardRunner(c, shard, "cpu", max_batch=8, max_ctx=64)
     stage = RingStage(runner, rank, world, P2PTransport(rank, world), split_head=split)
     assert stage.split == split
-    toks = _run(stage, 2)
+    toks = _run(stage, 2, model)
     stage.t.drain()
     dist.barrier()
     if stage.samples:
@@ -84,3 +84,28 @@ def test_two_rank_ring_matches_single_process(split):
     assert got == [r[:STEPS] for r in ref]
   else:
     assert got == ref
+
+
+def test_two_rank_ring_mixed_layer_model():
+  """The same ring with a model of differing layers: the fp32 residual stream travels between the ranks, each rank
+  keeps the state slots of its own recurrent layers, the scaled head stays whole on the last stage."""
+  model = "tiny-tarepel"
+  c = PRESETS[model]
+  full = ShardRunner(c, Shard(model, 0, c.num_layers - 1, c.num_layers), "cpu", max_batch=8, max_ctx=64)
+  from xotorch_support_jetson_amd.parallel.comm import LoopbackTransport
+  ref = _run(RingStage(full, 0, 1, LoopbackTransport(0, 1)), 2, model)
+  ctx = mp.get_context("spawn")
+  q = ctx.Queue()
+  port = _free_port()
+  procs = [ctx.Process(target=_worker, args=(r, 2, port, q, False, model)) for r in range(2)]
+  for p in procs:
+    p.start()
+  try:
+    got = q.get(timeout=240)
+  finally:
+    for p in procs:
+      p.join(timeout=60)
+      if p.is_alive():
+        p.kill()
+  assert all(p.exitcode == 0 for p in procs)
+  assert len(ref[0]) == STEPS + 1 and got == ref

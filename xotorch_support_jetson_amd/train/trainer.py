@@ -52,6 +52,8 @@ class ShardTrainer:
                weight_decay: float = 0.0, max_seq: int = 4096, grad_clip: float = 1.0):
     self.w = weights
     self.c: ModelConfig = weights.config
+    if self.c.is_mixed:
+      raise NotImplementedError(f"{self.c.model_type}: mixed-layer models are served, not trained, by this framework")
     self.shard = weights.shard
     self.device = torch.device(device)
     self.lr, self.betas, self.eps, self.wd = lr, betas, eps, weight_decay
