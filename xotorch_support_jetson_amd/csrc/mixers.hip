@@ -938,8 +938,10 @@ void attn_gated_chunk(const at::Tensor& q, const at::Tensor& k_cache, const at::
     const int hpg = (int)(H / G);
     int dpad = 16;
     while (dpad < d) dpad *= 2;
-    // key splits: enough workgroups to cover the chip (about two per CU), at least 64 keys each
-    int KS = (int)std::min<int64_t>(std::min<int64_t>(8, (chunk + 63) / 64), (512 + T * G - 1) / (T * G));
+    // key splits: enough workgroups to cover the chip (about four per CU), at least 64 keys each
+    // (64 tokens x 4 kv heads, about 530 keys each: 61 / 46 / 35 / 45 us when aiming at 256 / 512 / 1024 / 2048 workgroups)
+    const int64_t want_wgs = 1024;
+    int KS = (int)std::min<int64_t>(std::min<int64_t>(8, (chunk + 63) / 64), (want_wgs + T * G - 1) / (T * G));
     KS = std::max(KS, 1);
     at::Tensor part;
     if (KS > 1) part = at::empty({KS, T, H * d}, q.options().dtype(at::kFloat));
