@@ -4,7 +4,9 @@
 //   gelu_mul           gelu_tanh(gate) * up out of a fused projection's columns
 //   rope_kv_store      partial rotate-half RoPE on q and k, paged write of the rotated key and of the value
 //                      (the value may be the un-rotated key)
-//   attn_gated_chunk   chunk-local attention with sigmoid(score + bias[head]) weights, no normalisation
+//   attn_gated_chunk   chunk-local attention with sigmoid(score + bias[head]) weights, no normalisation: an MFMA
+//                      kernel for prompt portions (bf16), a (token, kv head, key split) kernel for single tokens
+//                      and fp32, a wave per (token, head) for groups above 8 query heads
 //   delta_prep         short causal convolutions + SiLU, unit-norm q / k, sigmoid write strength, scalar decay
 //   conv_state_update  the last taps-1 convolution inputs of every sequence -> its state slot
 //   gla_prep           per-key-channel decay sigmoid(low-rank z)^(1/tau)
@@ -134,8 +136,8 @@ __global__ void rope_kv_store_k(const float* __restrict__ P, int ldp, int q_off,
 // out[t, h * d + i] = out_scale * sum_j sigmoid(q.k_j * scale + pb[h]) v_j[i] over the keys j <= i's position of
 // the query's chunk.
 //
-// Simple kernel (any d <= 256, bf16 or fp32; single decoded tokens): one wave per (token, head), lanes over keys for
-// the scores, then lanes over value dims for the weighted sum.
+// Wave-per-(token, head) kernel (any d <= 256, bf16 or fp32; the fallback for more than 8 query heads per kv head):
+// lanes over keys for the scores, then lanes over value dims for the weighted sum.
 constexpr int ATT_TILE = 512;
 
 __device__ __forceinline__ void ld8(const float* p, float* o) {

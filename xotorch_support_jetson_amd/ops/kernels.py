@@ -469,7 +469,8 @@ def attn_gated_chunk(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, scal
   """out [T, H d] = out_scale * sum over the keys j <= i of query i's chunk (floor(i / chunk) == floor(j / chunk))
   of sigmoid(q_i . k_j * scale + pb[head]) v_j; positions count from each sequence's start.  Caches: K [pages, G, 64,
   d], V [pages, G, d, 64].  max_qlen: the step's longest run of new tokens of one sequence (0: unknown -> the total);
-  bf16 steps with runs above one token take the MFMA kernel, single tokens a wave per (token, head)."""
+  bf16 steps with runs above one token take the MFMA kernel; single tokens, fp32 and head sizes that are no
+  multiple of 32 a (token, kv head, key split) kernel that scores each key once for all query heads of its group."""
   _mix("attn_gated_chunk", _gpu(q))(q, k_cache, v_cache, block_tables, cu_q, ctx_lens, pb, float(scale), int(chunk),
                                     float(out_scale), out, int(max_qlen) or int(q.shape[0]))
 
