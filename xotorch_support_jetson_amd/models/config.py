@@ -49,20 +49,105 @@ class LinearRecurrenceSpec:
 
 
 @dataclass(frozen=True)
+class WindowAttnSpec:
+  """Softmax attention (GQA) over a sliding window plus pooled blocks: a query at position i sees the tokens j with
+  0 <= i - j < window (window 0: every earlier token) and, with pool > 0, one mean key / mean value per block of
+  `pool` tokens that ends at or before i - window; tokens, blocks and an optional per-head sink logit (no value) share
+  one softmax.  q / k / v may carry biases; rotate-half RoPE on the first rot_dims dims with optional wavelength-banded
+  frequency scaling rot_scaling = (factor, low, high, original); qk_norm divides q and k by their RMS per head after
+  the rotation.  kv_from >= 0: no key / value projections, the layer reads that layer's caches with its own queries
+  and its own window / pool."""
+  heads: int
+  kv_heads: int
+  dim: int
+  vdim: int
+  window: int
+  pool: int
+  rot_dims: int
+  rot_base: float
+  rot_scaling: Optional[tuple]
+  scale: float
+  qk_norm: bool = True
+  bias: bool = True
+  sink: bool = True
+  kv_from: int = -1
+
+
+@dataclass(frozen=True)
+class SSDSpec:
+  """State-space-duality recurrence (Mamba-2): per head a state S [state, vdim] in fp32,
+  S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x, with B / C shared by heads / groups heads, a causal
+  convolution of `conv` taps + SiLU over the x | B | C channels, dt = softplus(dt + bias); y is gated by silu(z) and
+  RMS-normed in norm_groups equal parts."""
+  heads: int
+  vdim: int
+  state: int
+  groups: int
+  conv: int
+  norm_groups: int = 1
+
+  @property
+  def inner(self) -> int:
+    return self.heads * self.vdim
+
+  @property
+  def conv_channels(self) -> int:
+    return self.inner + 2 * self.groups * self.state
+
+
+@dataclass(frozen=True)
+class FeedForwardSpec:
+  """A non-gated feed-forward W_down act(W_up h).  kind "polynorm": act(z) = a N(z) + b N(z^2) + c N(z^3) + e with N the
+  division of the token's ff vector by its RMS; kind "relu2_moe": `experts` experts with act = relu^2, the `top` largest
+  router logits chosen per token and weighted by the softmax over the chosen logits, plus (shared_ff > 0) one shared
+  expert of the same form scaled by a per-token sigmoid gate."""
+  kind: str  # polynorm | relu2_moe
+  ff: int
+  experts: int = 0
+  top: int = 0
+  shared_ff: int = 0
+
+
+@dataclass(frozen=True)
 class MixedLayerSpec:
-  """One layer of a model whose layers differ (ModelConfig.layer_specs): the token mixers that read the layer's
-  one normed input side by side, their output scales, and the gated feed-forward size (0: none)."""
+  """One layer of a model whose layers differ (ModelConfig.layer_specs).  Parallel blocks (ModelConfig.block
+  "parallel"): the token mixers attn / rec read the layer's one normed input side by side, with their output scales and
+  the gated feed-forward size ff (0: none).  Post-norm blocks ("postln"): one mixer, wattn or ssd, then the
+  feed-forward ffn (None: none)."""
   kind: str  # config.json's layer type
   attn: Optional[GatedAttnSpec] = None
   rec: Optional[LinearRecurrenceSpec] = None
   attn_scale: float = 1.0
   rec_scale: float = 1.0
   ff: int = 0
+  wattn: Optional[WindowAttnSpec] = None
+  ssd: Optional[SSDSpec] = None
+  ffn: Optional[FeedForwardSpec] = None
+
+  @property
+  def kv_dims(self) -> Optional[tuple]:
+    """(kv heads, key dim, value dim) of the paged K / V pool this layer owns (None: it has none of its own)."""
+    if self.attn is not None:
+      return self.attn.kv_heads, self.attn.dim, self.attn.dim
+    if self.wattn is not None and self.wattn.kv_from < 0:
+      return self.wattn.kv_heads, self.wattn.dim, self.wattn.vdim
+    return None
+
+  @property
+  def state_dims(self) -> Optional[tuple]:
+    """(heads, value dim, key dim, convolution taps, convolution channels) of the layer's recurrent state."""
+    if self.rec is not None:
+      r = self.rec
+      return r.heads, r.vdim, r.dim, r.conv, (2 * r.kv_heads * r.dim + r.heads * r.vdim) if r.conv > 0 else 0
+    if self.ssd is not None:
+      m = self.ssd
+      return m.heads, m.vdim, m.state, m.conv, m.conv_channels if m.conv > 0 else 0
+    return None
 
 
 @dataclass(frozen=True)
 class ModelConfig:
-  model_type: str  # llama | qwen2 | mistral | mixtral | tarepel
+  model_type: str  # llama | qwen2 | mistral | mixtral | ... | tarepel | mogelix
   vocab_size: int
   hidden_size: int
   intermediate_size: int
@@ -110,6 +195,10 @@ class ModelConfig:
   # an fp32 residual stream, scalar-gain RMS norms, per-channel layer scales, scaled logits
   layer_specs: Optional[tuple] = None
   logit_scale: float = 1.0
+  # block form of a mixed-layer model: "parallel" (Tarepel: pre-norm, mixers and feed-forward side by side) or "postln"
+  # (Mogelix: x <- norm(alpha x + gate * sublayer(x)) for the mixer, then for the feed-forward; per-channel norm weights)
+  block: str = "parallel"
+  postln_alpha: float = 1.0
 
   @property
   def is_mixed(self) -> bool:
@@ -118,7 +207,7 @@ class ModelConfig:
   @property
   def has_state(self) -> bool:
     """Some layer carries recurrent state per request (a state slot beside the KV pages)."""
-    return bool(self.layer_specs) and any(s.rec is not None for s in self.layer_specs)
+    return bool(self.layer_specs) and any(s.state_dims is not None for s in self.layer_specs)
 
   @property
   def qkv_size(self) -> int:
@@ -206,6 +295,23 @@ class ModelConfig:
 
 
 def mixed_layer_params(D: int, s: MixedLayerSpec) -> int:
+  if s.wattn is not None or s.ssd is not None:
+    n = 2 * D * (D + 1) + 2 * D  # the two sublayer gates and norms
+    if s.wattn is not None:
+      a = s.wattn
+      n += (D + 1) * a.heads * a.dim + a.heads * a.vdim * D + a.heads
+      if a.kv_from < 0:
+        n += (D + 1) * a.kv_heads * (a.dim + a.vdim)
+    if s.ssd is not None:
+      m = s.ssd
+      n += D * (2 * m.inner + 2 * m.groups * m.state + m.heads) + m.conv_channels * (m.conv + 1) + 3 * m.heads + \
+        m.inner + m.inner * D
+    f = s.ffn
+    if f is not None and f.kind == "polynorm":
+      n += 2 * D * f.ff + 4
+    elif f is not None:
+      n += f.experts * 2 * D * f.ff + f.experts * (D + 1) + (2 * D * f.shared_ff + D if f.shared_ff else 0)
+    return n
   n = 1 + 2 * D + 3 * D * s.ff
   if s.attn is not None:
     a = s.attn
@@ -282,9 +388,67 @@ def _tarepel_config(cfg: dict) -> ModelConfig:
     layer_specs=tuple(specs), logit_scale=float(cfg.get("logit_scale", 1.0)))
 
 
+def _mogelix_config(cfg: dict) -> ModelConfig:
+  """Mogelix config.json: {"architecture", "vocab", "width", "norm": {"eps"}, "postln_alpha", "layers": [{"type":
+  "attention" | "mamba2", "mixer": {...}, "mlp": {"kind": "dense", "ff"} | {"kind": "moe", "expert": {"ff"}, "router":
+  {"experts", "top"}, "shared": {"ff"}} | null}]}.  An attention mixer without "mask" sees every earlier token, without
+  "pool" no pooled blocks, without "rot" nothing is rotated; "kv_from": j borrows layer j's keys and values."""
+  specs = []
+  for i, L in enumerate(cfg["layers"]):
+    m, mlp = L["mixer"], L.get("mlp")
+    ffn = None
+    if mlp is not None:
+      kind = mlp.get("kind", "dense")
+      if kind == "dense":
+        ffn = FeedForwardSpec("polynorm", int(mlp["ff"]))
+      elif kind == "moe":
+        sh = mlp.get("shared")
+        ffn = FeedForwardSpec("relu2_moe", int(mlp["expert"]["ff"]), int(mlp["router"]["experts"]),
+                              int(mlp["router"]["top"]), int(sh["ff"]) if sh else 0)
+        if not 1 <= ffn.top <= ffn.experts:
+          raise ValueError(f"layer {i}: top {ffn.top} of {ffn.experts} experts")
+      else:
+        raise ValueError(f"layer {i}: unsupported feed-forward kind {kind!r}")
+    if L["type"] == "attention":
+      rot, mask = m.get("rot") or {}, m.get("mask") or {}
+      sc = rot.get("scaling")
+      scaling = (float(sc["factor"]), float(sc["low"]), float(sc["high"]), float(sc["original"])) if sc else None
+      src = m.get("kv_from")
+      a = WindowAttnSpec(int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"]), int(mask.get("size", 0)),
+                         int(mask.get("pool", 0)) if mask.get("size") else 0, int(rot.get("dims", 0)),
+                         float(rot.get("base", 10000.0)), scaling, float(m["scale"]), kv_from=-1 if src is None else int(src))
+      if a.heads % a.kv_heads or a.rot_dims % 2 or a.rot_dims > a.dim:
+        raise ValueError(f"layer {i}: heads {a.heads} / kv_heads {a.kv_heads} / rotary dims {a.rot_dims} do not fit")
+      if a.kv_from >= 0:
+        b = specs[a.kv_from].wattn if 0 <= a.kv_from < i else None
+        if b is None or b.kv_from >= 0 or (b.kv_heads, b.dim, b.vdim) != (a.kv_heads, a.dim, a.vdim):
+          raise ValueError(f"layer {i}: kv_from {a.kv_from} must name an earlier attention layer with projections of "
+                           "its own and the same key / value heads")
+      specs.append(MixedLayerSpec("attention", wattn=a, ffn=ffn))
+    elif L["type"] == "mamba2":
+      s = SSDSpec(int(m["heads"]), int(m["vdim"]), int(m["state"]), int(m.get("groups", 1)), int(m.get("conv", 1)),
+                  int(m.get("norm_groups", 1)))
+      if s.heads % s.groups or s.inner % s.norm_groups or s.conv < 1:
+        raise ValueError(f"layer {i}: heads {s.heads} / groups {s.groups} / norm_groups {s.norm_groups} do not fit")
+      specs.append(MixedLayerSpec("mamba2", ssd=s, ffn=ffn))
+    else:
+      raise ValueError(f"layer {i}: unknown layer type {L['type']!r}")
+  first = next((s.wattn for s in specs if s.wattn is not None), None)
+  return ModelConfig(
+    model_type="mogelix", vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]),
+    intermediate_size=max([s.ffn.ff for s in specs if s.ffn is not None] + [0]), num_layers=len(specs),
+    num_heads=first.heads if first else 1, num_kv_heads=first.kv_heads if first else 1,
+    head_dim=first.dim if first else 64, rms_norm_eps=float(cfg["norm"]["eps"]),
+    rope_theta=first.rot_base if first else 10000.0, max_position_embeddings=int(cfg.get("max_positions", 1 << 20)),
+    bos_token_id=int(cfg.get("bos_token_id", 0)), eos_token_ids=tuple(cfg.get("eos_token_ids", ())),
+    layer_specs=tuple(specs), block="postln", postln_alpha=float(cfg.get("postln_alpha", 1.0)))
+
+
 def from_hf_config(cfg: dict) -> ModelConfig:
   if cfg.get("architecture") == "Tarepel":
     return _tarepel_config(cfg)
+  if cfg.get("architecture") == "Mogelix":
+    return _mogelix_config(cfg)
   mt = cfg.get("model_type", "llama")
   if mt == "llava":
     return _llava_config(cfg)
@@ -513,6 +677,23 @@ TINY_TAREPEL = {
                "left_scale": 1.0, "right_scale": 0.5}},
   ]}
 PRESETS["tiny-tarepel"] = _tarepel_config(TINY_TAREPEL)
+_TINY_ROT = {"base": 10000.0, "dims": 16, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 64}}
+_TINY_MOE = {"kind": "moe", "expert": {"ff": 48}, "router": {"experts": 6, "top": 2}, "shared": {"ff": 64}}
+TINY_MOGELIX = {
+  "architecture": "Mogelix", "vocab": 288, "width": 96, "norm": {"eps": 1e-5}, "postln_alpha": 1.5,
+  "layers": [
+    {"type": "mamba2", "mlp": {"kind": "dense", "ff": 160},
+     "mixer": {"heads": 4, "vdim": 16, "state": 24, "groups": 2, "conv": 3, "norm_groups": 2}},
+    {"type": "attention", "mlp": _TINY_MOE,
+     "mixer": {"heads": 6, "kv_heads": 2, "dim": 32, "vdim": 16, "mask": {"size": 20, "pool": 5}, "rot": _TINY_ROT,
+               "scale": 0.3}},
+    {"type": "attention", "mlp": None,
+     "mixer": {"heads": 6, "kv_heads": 2, "dim": 32, "vdim": 16, "kv_from": 1, "mask": {"size": 9, "pool": 3},
+               "rot": _TINY_ROT, "scale": 0.25}},
+    {"type": "mamba2", "mlp": _TINY_MOE,
+     "mixer": {"heads": 2, "vdim": 32, "state": 16, "groups": 1, "conv": 4, "norm_groups": 1}},
+  ]}
+PRESETS["tiny-mogelix"] = _mogelix_config(TINY_MOGELIX)
 # aliases of the reference's model cards that share an architecture
 for _alias, _base in {"llama-3.1-70b-bf16": "llama-3.1-70b", "nemotron-70b": "llama-3.1-70b",
                       "deepseek-r1-distill-llama-70b": "llama-3.1-70b", "deepseek-r1-distill-llama-8b": "llama-3.1-8b",

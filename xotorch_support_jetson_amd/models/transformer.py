@@ -98,11 +98,34 @@ class KVCache:
       # one K [pages, G, 64, d] and one V [pages, G, d, 64] pool per layer that has an attention mixer (None for the others):
       # layers may differ in heads and sizes; the value pool holds whatever the layer's mixer stores as values
       ids = list(layer_ids) if layer_ids is not None else list(range(n_layers))
-      specs = [c.layer_specs[i].attn for i in ids]
-      self.k = [None if a is None else torch.zeros(num_pages, a.kv_heads, PAGE, a.dim, device=device, dtype=dtype)
-                for a in specs]
-      self.v = [None if a is None else torch.zeros(num_pages, a.kv_heads, a.dim, PAGE, device=device, dtype=dtype)
-                for a in specs]
+      dims = [c.layer_specs[i].kv_dims for i in ids]
+      self.k = [None if a is None else torch.zeros(num_pages, a[0], PAGE, a[1], device=device, dtype=dtype) for a in dims]
+      self.v = [None if a is None else torch.zeros(num_pages, a[0], a[2], PAGE, device=device, dtype=dtype) for a in dims]
+      # window attention with pooled blocks: per layer the (source layer, block size) pooled caches it reads, K
+      # [pages, G, per, d] and V [pages, G, dv, per8]; entries live with the page of a block's last token, so they are
+      # handed out and returned with the sequence's pages.  pool_owner[j]: this layer fills them (the first layer of
+      # the shard that reads this source with this block size); a layer that borrows another's keys and values aliases
+      # that layer's pools.
+      self.kp: List[Optional[torch.Tensor]] = [None] * len(ids)
+      self.vp: List[Optional[torch.Tensor]] = [None] * len(ids)
+      self.pool_owner = [False] * len(ids)
+      made = {}
+      for j, i in enumerate(ids):
+        a = c.layer_specs[i].wattn
+        if a is None:
+          continue
+        src = i if a.kv_from < 0 else a.kv_from
+        if src not in ids:
+          raise ValueError(f"layer {i} reads the keys and values of layer {src}, which is not on this shard")
+        js = ids.index(src)
+        self.k[j], self.v[j] = self.k[js], self.v[js]
+        if a.pool > 0 and a.window > 0:
+          if (src, a.pool) not in made:
+            per, per8 = K.pool_dims(a.pool)
+            made[(src, a.pool)] = (torch.zeros(num_pages, a.kv_heads, per, a.dim, device=device, dtype=dtype),
+                                   torch.zeros(num_pages, a.kv_heads, a.vdim, per8, device=device, dtype=dtype))
+            self.pool_owner[j] = True
+          self.kp[j], self.vp[j] = made[(src, a.pool)]
       return
     if c.is_mla:
       self.k = torch.zeros(n_layers, num_pages, PAGE, c.mla_dim, device=device, dtype=dtype)
@@ -115,15 +138,28 @@ class KVCache:
   def bytes_per_page(c: ModelConfig, n_layers: int, layer_ids=None, itemsize: int = 2) -> int:
     if c.is_mixed:
       ids = list(layer_ids) if layer_ids is not None else list(range(n_layers))
-      return max(1, sum(2 * a.kv_heads * PAGE * a.dim * itemsize for a in (c.layer_specs[i].attn for i in ids)
-                        if a is not None))
+      n, seen = 0, set()
+      for i in ids:
+        a, w = c.layer_specs[i].kv_dims, c.layer_specs[i].wattn
+        if a is not None:
+          n += a[0] * PAGE * (a[1] + a[2]) * itemsize
+        if w is not None and w.pool > 0 and w.window > 0 and (w.kv_from if w.kv_from >= 0 else i, w.pool) not in seen:
+          seen.add((w.kv_from if w.kv_from >= 0 else i, w.pool))
+          per, per8 = K.pool_dims(w.pool)
+          n += w.kv_heads * (per * w.dim + per8 * w.vdim) * itemsize
+      return max(1, n)
     if c.is_mla:
       return n_layers * PAGE * c.mla_dim * 2
     return 2 * n_layers * c.num_kv_heads * PAGE * c.head_dim * 2
 
   def nbytes(self) -> int:
-    ts = (self.k + self.v) if isinstance(self.k, list) else (self.k, self.v)
-    return sum(t.numel() * t.element_size() for t in ts if t is not None)
+    ts = (self.k + self.v + getattr(self, "kp", []) + getattr(self, "vp", [])) if isinstance(self.k, list) else (self.k, self.v)
+    seen, n = set(), 0
+    for t in ts:
+      if t is not None and t.data_ptr() not in seen:
+        seen.add(t.data_ptr())
+        n += t.numel() * t.element_size()
+    return n
 
 
 class StatePool:
@@ -136,10 +172,10 @@ class StatePool:
     self.S: List[Optional[torch.Tensor]] = []
     self.conv: List[Optional[torch.Tensor]] = []
     for i in layer_ids:
-      r = c.layer_specs[i].rec
-      self.S.append(None if r is None else torch.zeros(slots, r.heads, r.vdim, r.dim, device=device, dtype=torch.float32))
-      ch = 0 if r is None or r.conv <= 0 else 2 * r.kv_heads * r.dim + r.heads * r.vdim
-      self.conv.append(torch.zeros(slots, max(r.conv - 1, 0), ch, device=device, dtype=torch.float32) if ch else None)
+      sd = c.layer_specs[i].state_dims  # (heads, value dim, key dim, taps, convolution channels)
+      self.S.append(None if sd is None else torch.zeros(slots, sd[0], sd[1], sd[2], device=device, dtype=torch.float32))
+      self.conv.append(torch.zeros(slots, max(sd[3] - 1, 0), sd[4], device=device, dtype=torch.float32)
+                       if sd is not None and sd[4] else None)
 
   def clear(self, slot: int) -> None:
     for t in self.S + self.conv:
@@ -166,11 +202,17 @@ class ShardModel:
       self.head_rows, self._head_cache = None, None
       # one [rows, R] (cos | sin) table per distinct (rotary dims, base) among the attention mixers
       self.rope_tabs = {}
+      from ..ops.rope import build_cos_sin
       for i in self.layer_ids:
         a = c.layer_specs[i].attn
         if a is not None and a.rot_dims and (a.rot_dims, a.rot_base) not in self.rope_tabs:
-          from ..ops.rope import build_cos_sin
           self.rope_tabs[(a.rot_dims, a.rot_base)] = build_cos_sin(a.rot_dims, self.rope_rows, a.rot_base, None, self.device)
+        a = c.layer_specs[i].wattn
+        if a is not None and a.rot_dims and (a.rot_dims, a.rot_base, a.rot_scaling) not in self.rope_tabs:
+          sc = a.rot_scaling and dict(rope_type="llama3", factor=a.rot_scaling[0], low_freq_factor=a.rot_scaling[1],
+                                      high_freq_factor=a.rot_scaling[2], original_max_position_embeddings=a.rot_scaling[3])
+          self.rope_tabs[(a.rot_dims, a.rot_base, a.rot_scaling)] = build_cos_sin(a.rot_dims, self.rope_rows, a.rot_base,
+                                                                                 sc, self.device)
       return
     self.scale = 1.0 / math.sqrt(c.head_dim)
     max_pos = max(max_ctx, 16)
@@ -442,6 +484,8 @@ class ShardModel:
     n = len(self.layer_ids)
     last = self.shard.is_last_layer()
     adt = (w.layers[self.layer_ids[0]].in_w if n else w.lm_head).dtype
+    if c.block == "postln":
+      return self._forward_postln(h, inp, adt)
     bufs = {}
 
     def rows(name: str, live: int, padded: int) -> torch.Tensor:
@@ -479,6 +523,140 @@ class ShardModel:
     K.resid_scale_norm(hl, gain=w.norm, eps=c.rms_norm_eps, out=xn)
     logits = self._proj(xn, w.lm_head)[:, :c.vocab_size]
     return logits * c.logit_scale
+
+  # ------------------------------------------------------------------ post-norm blocks (window attention / SSD, MoE)
+  def _window_attn(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:
+    """Softmax attention over a sliding window, pooled blocks before it and a sink: biases + RoPE + per-head RMS
+    division + paged write, the pooled caches' update for blocks that this step completed, then the attention."""
+    a = lw.spec.wattn
+    q = torch.empty(P.shape[0], a.heads, a.dim, dtype=mix.dtype, device=P.device)
+    tab = self.rope_tabs.get((a.rot_dims, a.rot_base, a.rot_scaling))
+    own = a.kv_from < 0
+    K.qk_norm_rope_store(P, lw.in_b, lw.cols["q"][0], lw.cols["k"][0] if own else -1, lw.cols["v"][0] if own else -1,
+                         a.heads, a.kv_heads, a.dim, a.vdim, a.rot_dims if tab is not None else 0, inp.positions,
+                         tab if tab is not None else torch.zeros(1, 0, device=P.device), inp.slots, self.c.rms_norm_eps,
+                         a.qk_norm, q, self.kv.k[j], self.kv.v[j])
+    if self.kv.pool_owner[j]:
+      K.kv_pool_update(self.kv.k[j], self.kv.v[j], self.kv.kp[j], self.kv.vp[j], inp.block_tables, inp.cu_q, inp.ctx_lens,
+                       a.pool, inp.max_qlen)
+    pool = a.pool if self.kv.kp[j] is not None else 0
+    K.attn_window_pool(q, self.kv.k[j], self.kv.v[j], self.kv.kp[j], self.kv.vp[j], inp.block_tables, inp.cu_q,
+                       inp.ctx_lens, lw.sink, a.scale, a.window, pool, mix[:, :a.heads * a.vdim], max_qlen=inp.max_qlen)
+
+  def _ssd(self, P: torch.Tensor, lw, j: int, inp: StepInputs, mix: torch.Tensor) -> None:
+    """Mamba-2 mixer on the state slots: convolution + SiLU, step sizes and decays, the recurrence on the fp32 state
+    (the framework's linear recurrence with one decay per head: q = C, k = B, v = dt x), skip, gate, grouped norm."""
+    m, st, dev = lw.spec.ssd, self.state, P.device
+    T = P.shape[0]
+    inner, gn = m.inner, m.groups * m.state
+    xbc = torch.empty(T, m.conv_channels, dtype=torch.float32, device=dev)
+    v = torch.empty(T, inner, dtype=torch.float32, device=dev)
+    decay = torch.empty(T, m.heads, dtype=torch.float32, device=dev)
+    o = torch.empty(T, inner, dtype=torch.float32, device=dev)
+    i0 = lw.cols["in"][0]
+    K.ssd_prep(P, i0 + inner, i0 + 2 * inner + 2 * gn, lw.conv_w, lw.conv_b, st.conv[j], inp.state_slots, inp.cu_q,
+               lw.A_log, lw.dt_bias, m.heads, m.vdim, xbc, v, decay)
+    K.linear_recurrence(xbc[:, inner + gn:], xbc[:, inner:inner + gn], v, decay, None, 1.0, st.S[j], inp.state_slots,
+                        inp.cu_q, o)
+    K.ssd_gate_norm(o, xbc, lw.skip_d, P, i0, lw.ssd_norm, m.norm_groups, self.c.rms_norm_eps, mix)
+
+  def _relu2_moe(self, hn: torch.Tensor, P: torch.Tensor, lw, rows) -> torch.Tensor:
+    """Routed relu^2 experts + the gated shared expert -> fp32 [T, D].  Routing on the framework's top-k kernel (the
+    softmax over the chosen logits), experts on the grouped GEMMs (bf16) or per expert on the vendor SGEMM (fp32)."""
+    f, dev = lw.spec.ffn, P.device
+    T, D = hn.shape[0], self.c.hidden_size
+    E, k = f.experts, f.top
+    r0 = lw.ff_cols["router"][0]
+    logits = (P[:, r0:r0 + E] + lw.router_b).contiguous()
+    if P.is_cuda:
+      topw = torch.empty(T * k, dtype=torch.float32, device=dev)
+      topi, slot_of, sorted_tok = (torch.empty(T * k, dtype=torch.int32, device=dev) for _ in range(3))
+      off = torch.empty(E + 1, dtype=torch.int32, device=dev)
+      if E <= 64 and k <= 8:
+        require().moe_route(logits, k, topw, topi, slot_of, sorted_tok, off)
+      else:
+        K.moe_route_ds(logits, None, k, 1, 1, 0, False, True, 1.0, outs=(topw, topi, slot_of, sorted_tok, off))
+    else:
+      val, idx = torch.topk(logits, k, dim=-1)
+      topw, topi = torch.softmax(val, -1).reshape(-1), idx.reshape(-1).int()
+      order = torch.argsort(topi, stable=True)
+      slot_of = torch.empty_like(order)
+      slot_of[order] = torch.arange(T * k)
+      sorted_tok = (order // k).int()
+      off = torch.cat([torch.zeros(1, dtype=torch.long), torch.bincount(topi.long(), minlength=E).cumsum(0)]).int()
+    Fp = lw.ex_up_w.shape[1]
+    if hn.dtype == torch.bfloat16 and hn.is_cuda:
+      C = require()
+      up = torch.empty(T * k, Fp, dtype=torch.float32, device=dev)
+      C.gemm_moe(hn, lw.ex_up_w, up, off, sorted_tok, K.EPI["none"], T, layout_of(lw.ex_up_w) == "stream", 1, 0)
+      act = torch.empty(T * k, Fp, dtype=torch.bfloat16, device=dev)
+      K.relu2(up, 0, Fp, act)
+      y = torch.empty(T * k, lw.ex_down_w.shape[1], dtype=torch.float32, device=dev)
+      C.gemm_moe(act, lw.ex_down_w, y, off, None, K.EPI["none"], T, layout_of(lw.ex_down_w) == "stream", 1, 0)
+    else:
+      # all-fp32 run: one vendor SGEMM pair per expert that has rows (the offsets come to the host)
+      y = torch.zeros(T * k, lw.ex_down_w.shape[1], dtype=torch.float32, device=dev)
+      offs = off.tolist()
+      for e in range(E):
+        if offs[e + 1] > offs[e]:
+          xe = hn.index_select(0, sorted_tok[offs[e]:offs[e + 1]].long()).float()
+          y[offs[e]:offs[e + 1]] = torch.relu(xe @ lw.ex_up_w[e].float().t()).pow(2) @ lw.ex_down_w[e].float().t()
+    sh_y = None
+    if f.shared_ff:
+      act = rows("sh_act", f.shared_ff, lw.down_w.shape[1])
+      K.relu2(P, lw.ff_cols["sh_up"][0], f.shared_ff, act)
+      sh_y = self._proj(act, lw.down_w)
+    out = torch.empty(T, D, dtype=torch.float32, device=dev)
+    K.moe_weighted_sum(y, slot_of, topw, k, sh_y, P, lw.ff_cols["sh_gate"][0] if f.shared_ff else 0, out)
+    return out
+
+  def _forward_postln(self, h: torch.Tensor, inp: StepInputs, adt) -> torch.Tensor:
+    """Layers of post-norm blocks on the fp32 stream h (hn: its copy in the GEMMs' operand dtype):
+      P = hn @ in_w^T                              the mixer's input projections and the mixer gate in one GEMM
+      h <- norm1(alpha h + sigmoid(gate + b) * (mixer(P) @ out_w^T))
+      P = hn @ ff_w^T                              feed-forward up (or router, shared up, shared gate) and its gate
+      h <- norm2(alpha h + sigmoid(gate + b) * ff(P))
+    Returns h (non-last shard) or head(norm(h rows inp.last_idx))."""
+    c, w = self.c, self.w
+    T, D = h.shape
+    Dp = -(-D // 128) * 128
+    bufs = {}
+
+    def rows(name: str, live: int, padded: int) -> torch.Tensor:
+      key = (name, live, padded)
+      if key not in bufs:
+        bufs[key] = (torch.zeros if padded > live else torch.empty)(T, padded, dtype=adt, device=h.device)
+      return bufs[key]
+    hn = rows("hn", D, Dp)
+    hn[:, :D] = h.to(adt)
+    for j, li in enumerate(self.layer_ids):
+      lw = w.layers[li]
+      s = lw.spec
+      P = self._proj(hn, lw.in_w)
+      mix = rows("mix", lw.mix_cols["mix"][1], lw.out_w.shape[1])
+      if s.wattn is not None:
+        self._window_attn(P, lw, j, inp, mix)
+      else:
+        self._ssd(P, lw, j, inp, mix)
+      y = self._proj(mix, lw.out_w)
+      K.gated_postnorm(h, y, P, lw.cols["gate"][0], lw.gate1_b, c.postln_alpha, lw.norm1, c.rms_norm_eps, hn)
+      f = s.ffn
+      if f is None:
+        continue
+      P = self._proj(hn, lw.ff_w)
+      if f.kind == "polynorm":
+        act = rows("act", f.ff, lw.down_w.shape[1])
+        K.polynorm_act(P, lw.ff_cols["up"][0], f.ff, lw.act, c.rms_norm_eps, act)
+        y = self._proj(act, lw.down_w)
+      else:
+        y = self._relu2_moe(hn, P, lw, rows)
+      K.gated_postnorm(h, y, P, lw.ff_cols["gate"][0], lw.gate2_b, c.postln_alpha, lw.norm2, c.rms_norm_eps, hn)
+    if not self.shard.is_last_layer():
+      return h
+    hl = h.index_select(0, inp.last_idx)
+    xn = torch.zeros(hl.shape[0], Dp, dtype=adt, device=h.device)
+    K.gated_postnorm(hl, None, None, 0, None, 1.0, w.norm, c.rms_norm_eps, xn)
+    return self._proj(xn, w.lm_head)[:, :c.vocab_size]
 
   # ------------------------------------------------------------------ forward
   @torch.inference_mode()

@@ -336,7 +336,7 @@ def prepare_for_decode(sw: "ShardWeights", keep_rowmajor: Iterable[str] = (), fp
   if sw.config.is_mixed:  # fused projections of mixed-layer models (bf16 runs; an fp32 run keeps vendor SGEMM layouts)
     for lw in sw.layers.values():
       if lw.in_w.dtype == torch.bfloat16:
-        lw.in_w, lw.out_w, lw.down_w = conv(lw.in_w), conv(lw.out_w), conv(lw.down_w)
+        lw.in_w, lw.out_w, lw.down_w, lw.ff_w = conv(lw.in_w), conv(lw.out_w), conv(lw.down_w), conv(lw.ff_w)
     if sw.lm_head is not None and sw.lm_head.dtype == torch.bfloat16:
       sw.lm_head = conv(sw.lm_head)
     return sw
@@ -682,8 +682,8 @@ class MixedLayerWeights:
   cols: Dict[str, tuple]
   out_w: torch.Tensor
   mix_cols: Dict[str, tuple]  # "attn" / "rec": (offset, size) in the mixers' output row
-  norm_g: torch.Tensor  # [1] fp32
-  ls1: torch.Tensor  # [D] fp32
+  norm_g: Optional[torch.Tensor] = None  # [1] fp32 (parallel blocks)
+  ls1: Optional[torch.Tensor] = None  # [D] fp32
   ls2: Optional[torch.Tensor] = None
   down_w: Optional[torch.Tensor] = None
   attn_pb: Optional[torch.Tensor] = None  # [H] fp32
@@ -694,6 +694,25 @@ class MixedLayerWeights:
   a2_w: Optional[torch.Tensor] = None  # [H d, rank] fp32
   a2_b: Optional[torch.Tensor] = None
   router: Optional[torch.Tensor] = None  # (dense feed-forward only; kept for code that asks)
+  # post-norm blocks (config.block "postln"): `in_w` = [the mixer's input projections | the mixer gate], a second
+  # fused projection `ff_w` = [feed-forward up (or router | shared up | shared gate) | the feed-forward gate] reads the
+  # stream after the first norm (`ff_cols` addresses its result); out_w is the mixer's output projection, down_w the
+  # dense (or shared expert's) down projection
+  norm1: Optional[torch.Tensor] = None  # [D] fp32 weights of the norms after the mixer / the feed-forward
+  norm2: Optional[torch.Tensor] = None
+  gate1_b: Optional[torch.Tensor] = None  # [D] fp32 biases of the sublayer gates
+  gate2_b: Optional[torch.Tensor] = None
+  in_b: Optional[torch.Tensor] = None  # [in_w rows] fp32: q / k / v biases at their columns, zero elsewhere
+  sink: Optional[torch.Tensor] = None  # [H] fp32
+  conv_b: Optional[torch.Tensor] = None  # [C] fp32
+  skip_d: Optional[torch.Tensor] = None  # [H] fp32 (SSD: D)
+  ssd_norm: Optional[torch.Tensor] = None  # [inner] fp32
+  ff_w: Optional[torch.Tensor] = None
+  ff_cols: Optional[Dict[str, tuple]] = None
+  act: Optional[torch.Tensor] = None  # [4] fp32 PolyNorm coefficients
+  router_b: Optional[torch.Tensor] = None  # [E] fp32
+  ex_up_w: Optional[torch.Tensor] = None  # [E, Fp, Dp] experts' up projections
+  ex_down_w: Optional[torch.Tensor] = None  # [E, Dq, Fp]
 
   def tensors(self) -> Dict[str, torch.Tensor]:
     return {k: v for k, v in self.__dict__.items() if isinstance(v, torch.Tensor)}
@@ -753,8 +772,124 @@ def build_mixed_layer(spec, get, p: str, D: int, device, dtype) -> MixedLayerWei
   return lw
 
 
+def _fused_rows(blocks, D: int, row_mult: int = 64):
+  """[(name, [n_i, D] tensor)] -> (zero-padded [Np, Dp] matrix, {name: (row offset, rows)})."""
+  cols, off = {}, 0
+  for n, w in blocks:
+    cols[n] = (off, w.shape[0])
+    off += w.shape[0]
+  m = torch.zeros(_up(max(off, 1), row_mult), _up(D, 128))
+  if off:
+    m[:off, :D] = torch.cat([w for _, w in blocks], 0)
+  return m, cols
+
+
+def _pad2(w: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
+  out = torch.zeros(rows, cols)
+  out[:w.shape[0], :w.shape[1]] = w
+  return out
+
+
+def build_postln_layer(spec, get, p: str, D: int, device, dtype) -> MixedLayerWeights:
+  """One post-norm layer (window attention or SSD mixer, PolyNorm or relu^2-MoE feed-forward) from `get(name)`."""
+  def dev(t, dt=torch.float32):
+    return t.to(device=device, dtype=dt).contiguous()
+  m = p + "mix."
+  a, sd, f = spec.wattn, spec.ssd, spec.ffn
+  blocks, bias = [], {}
+  if a is not None:
+    names = ["q"] if a.kv_from >= 0 else ["q", "k", "v"]
+    blocks = [(n, get(m + n)) for n in names]
+    if a.bias:
+      bias = {n: get(m + n + ".b") for n in names}
+    out = get(m + "o")
+  else:
+    blocks = [("in", get(m + "in"))]
+    out = get(m + "o")
+  blocks.append(("gate", get(p + "rg1")))
+  in_w, cols = _fused_rows(blocks, D)
+  lw = MixedLayerWeights(spec, dev(in_w, dtype), cols, dev(_pad2(out, _up(D, 64), _up(out.shape[1], 128)), dtype),
+                         {"mix": (0, out.shape[1])})
+  lw.norm1, lw.gate1_b = dev(get(p + "norm1")), dev(get(p + "rg1.b"))
+  if bias:
+    b = torch.zeros(in_w.shape[0])
+    for n, t in bias.items():
+      b[cols[n][0]:cols[n][0] + cols[n][1]] = t
+    lw.in_b = dev(b)
+  if a is not None and a.sink:
+    lw.sink = dev(get(m + "sink"))
+  if sd is not None:
+    lw.conv_w, lw.conv_b = dev(get(m + "conv")), dev(get(m + "conv.b"))
+    lw.A_log, lw.dt_bias, lw.skip_d = dev(get(m + "A_log")), dev(get(m + "dt_bias")), dev(get(m + "D"))
+    lw.ssd_norm = dev(get(m + "norm"))
+  if f is None:
+    return lw
+  q = p + "mlp."
+  if f.kind == "polynorm":
+    fb = [("up", get(q + "up"))]
+    down = get(q + "down")
+    lw.act = dev(get(q + "act"))
+  else:
+    fb = [("router", get(q + "router"))]
+    down = None
+    if f.shared_ff:
+      fb += [("sh_up", get(q + "shared.up")), ("sh_gate", get(q + "shared.sg").reshape(1, D))]
+      down = get(q + "shared.down")
+    lw.router_b = dev(get(q + "router.b"))
+    Fp, Dp = _up(f.ff, 128), _up(D, 128)
+    lw.ex_up_w = dev(torch.stack([_pad2(get(q + f"e{e}.up"), Fp, Dp) for e in range(f.experts)]), dtype)
+    lw.ex_down_w = dev(torch.stack([_pad2(get(q + f"e{e}.down"), Dp, Fp) for e in range(f.experts)]), dtype)
+  fb.append(("gate", get(p + "rg2")))
+  ff_w, lw.ff_cols = _fused_rows(fb, D)
+  lw.ff_w = dev(ff_w, dtype)
+  if down is not None:
+    lw.down_w = dev(_pad2(down, _up(D, 64), _up(down.shape[1], 128)), dtype)
+  lw.norm2, lw.gate2_b = dev(get(p + "norm2")), dev(get(p + "rg2.b"))
+  return lw
+
+
+def postln_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
+  """Name -> shape of every tensor of a post-norm mixed-layer checkpoint (Mogelix)."""
+  D, out = c.hidden_size, {}
+  out["embed"] = (c.vocab_size, D)
+  for i, s in enumerate(c.layer_specs):
+    p, m = f"l{i}.", f"l{i}.mix."
+    out[p + "norm1"], out[p + "rg1"], out[p + "rg1.b"] = (D,), (D, D), (D,)
+    a, sd, f = s.wattn, s.ssd, s.ffn
+    if a is not None:
+      proj = [("q", a.heads * a.dim)] + ([("k", a.kv_heads * a.dim), ("v", a.kv_heads * a.vdim)] if a.kv_from < 0 else [])
+      for n, rows in proj:
+        out[m + n] = (rows, D)
+        if a.bias:
+          out[m + n + ".b"] = (rows,)
+      if a.sink:
+        out[m + "sink"] = (a.heads,)
+      out[m + "o"] = (D, a.heads * a.vdim)
+    if sd is not None:
+      out[m + "in"] = (2 * sd.inner + 2 * sd.groups * sd.state + sd.heads, D)
+      out[m + "conv"], out[m + "conv.b"] = (sd.conv_channels, sd.conv), (sd.conv_channels,)
+      out[m + "dt_bias"], out[m + "A_log"], out[m + "D"] = (sd.heads,), (sd.heads,), (sd.heads,)
+      out[m + "norm"], out[m + "o"] = (sd.inner,), (D, sd.inner)
+    if f is None:
+      continue
+    q = p + "mlp."
+    out[p + "norm2"], out[p + "rg2"], out[p + "rg2.b"] = (D,), (D, D), (D,)
+    if f.kind == "polynorm":
+      out[q + "up"], out[q + "down"], out[q + "act"] = (f.ff, D), (D, f.ff), (4,)
+    else:
+      for e in range(f.experts):
+        out[q + f"e{e}.up"], out[q + f"e{e}.down"] = (f.ff, D), (D, f.ff)
+      out[q + "router"], out[q + "router.b"] = (f.experts, D), (f.experts,)
+      if f.shared_ff:
+        out[q + "shared.up"], out[q + "shared.down"], out[q + "shared.sg"] = (f.shared_ff, D), (D, f.shared_ff), (1, D)
+  out["final.norm"], out["head"] = (D,), (c.vocab_size, D)
+  return out
+
+
 def mixed_tensor_shapes(c: ModelConfig) -> Dict[str, tuple]:
   """Name -> shape of every tensor of a mixed-layer checkpoint (random init, checkpoint validation)."""
+  if c.block == "postln":
+    return postln_tensor_shapes(c)
   D, out = c.hidden_size, {}
   out["embed"] = (c.vocab_size, D)
   for i, s in enumerate(c.layer_specs):
@@ -791,7 +926,9 @@ def random_mixed_tensors(c: ModelConfig, seed: int = 0) -> Dict[str, torch.Tenso
     leaf = name.split(".")[-1]
     if name.endswith(".conv"):
       t = torch.randn(shape, generator=g) * 0.5
-    elif leaf in ("norm1",) or name == "final.norm":
+    elif leaf in ("sink", "D", "act") or (leaf == "b" and c.block == "postln"):
+      t = torch.randn(shape, generator=g) * (0.5 if leaf == "b" else 1.0)
+    elif leaf in ("norm1", "norm2") or name == "final.norm":
       t = 1.0 + 0.1 * torch.randn(shape, generator=g)
     elif leaf in ("ls1", "ls2"):
       t = 0.5 + 0.1 * torch.randn(shape, generator=g)
@@ -815,12 +952,13 @@ def mixed_weights(c: ModelConfig, shard: Shard, get, device, dtype) -> ShardWeig
   """ShardWeights of a mixed-layer model from `get(name) -> fp32 CPU tensor`."""
   sw = ShardWeights(c, shard)
   D = c.hidden_size
+  build = build_postln_layer if c.block == "postln" else build_mixed_layer
   for i in shard.layers():
-    sw.layers[i] = build_mixed_layer(c.layer_specs[i], get, f"l{i}.", D, device, dtype)
+    sw.layers[i] = build(c.layer_specs[i], get, f"l{i}.", D, device, dtype)
   if shard.is_first_layer():
     sw.embed = get("embed").to(device=device, dtype=torch.float32).contiguous()  # gathered into the fp32 residual
   if shard.is_last_layer():
-    sw.norm = get("final.norm").reshape(1).to(device=device, dtype=torch.float32)
+    sw.norm = get("final.norm").reshape(-1).to(device=device, dtype=torch.float32)
     head = torch.zeros(_up(c.vocab_size, 64), _up(D, 128))
     head[:c.vocab_size, :D] = get("head")
     sw.lm_head = head.to(device=device, dtype=dtype).contiguous()
@@ -828,8 +966,8 @@ def mixed_weights(c: ModelConfig, shard: Shard, get, device, dtype) -> ShardWeig
 
 
 def load_mixed_weights(model_dir: Path, c: ModelConfig, shard: Shard, device, dtype) -> ShardWeights:
-  """Tarepel checkpoint (flat names: embed, l<i>.norm1, l<i>.mix.*, l<i>.mlp.*, l<i>.ls1 / ls2, final.norm, head).
-  The decay rank of a gated-linear-attention layer is the a1 tensor's row count."""
+  """Tarepel / Mogelix checkpoint (flat names: embed, l<i>.norm1, l<i>.mix.*, l<i>.mlp.*, l<i>.ls1 / ls2 or l<i>.rg1 /
+  rg2, final.norm, head).  The decay rank of a gated-linear-attention layer is the a1 tensor's row count."""
   from safetensors import safe_open
   wm = _weight_map(Path(model_dir))
   handles = {}

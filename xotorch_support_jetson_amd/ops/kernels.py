@@ -497,3 +497,66 @@ def linear_recurrence(q, k, v, decay, beta, q_scale: float, state, state_slots, 
 def gated_rmsnorm(o, w, P, g_off: int, eps: float, out_scale: float, out) -> None:
   """out [T, H dv] = o / rms(o per head) * w * silu(P[:, g_off : +H dv]) * out_scale."""
   _mix("gated_rmsnorm", _gpu(o))(o, w, P, int(g_off), float(eps), float(out_scale), out)
+
+
+# ------------------------------------------------------------------ post-norm blocks (csrc/hybrid.hip)
+pool_dims = ref.pool_dims
+
+
+def gated_postnorm(x, y, P, g_off: int, gate_b, alpha: float, w, eps: float, out=None) -> None:
+  """fp32 stream rows x [T, D] <- (alpha x + y * sigmoid(P[:, g_off : +D] + gate_b)) / rms * w in place (P None: the
+  sublayer's result y is not gated); with `out`, out[:, :D] = the new x in out's dtype (the next GEMM's operand)."""
+  _mix("gated_postnorm", _gpu(x))(x, y, P, int(g_off), gate_b, float(alpha), w, float(eps), out)
+
+
+def qk_norm_rope_store(P, bias, q_off: int, k_off: int, v_off: int, H: int, G: int, d: int, dv: int, R: int, pos, cos_sin,
+                       slots, eps: float, qk_norm: bool, q_out, k_cache, v_cache) -> None:
+  """q / k / v = P's columns (+ bias, one fp32 number per column of P); rotate-half RoPE on the first R dims of every
+  q / k head, then (qk_norm) each head divided by its RMS; q -> q_out [T, H, d], k -> k_cache [pages, G, 64, d],
+  v -> v_cache [pages, G, dv, 64] at `slots`.  k_off < 0: the layer has no keys and values of its own."""
+  _mix("qk_norm_rope_store", _gpu(P))(P, bias, int(q_off), int(k_off), int(v_off), int(H), int(G), int(d), int(dv), int(R),
+                                      pos, cos_sin, slots, float(eps), bool(qk_norm), q_out, k_cache, v_cache)
+
+
+def kv_pool_update(k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, pool: int, max_qlen: int) -> None:
+  """Mean key and value of every block of `pool` consecutive tokens whose last token is among the step's new ones,
+  read from the paged caches as they hold them, into the pooled caches kp [pages, G, per, d] / vp [pages, G, dv, per8]
+  (entry of block b: with the page of its last token, see pool_dims)."""
+  _mix("kv_pool_update", _gpu(k_cache))(k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, int(pool), int(max_qlen))
+
+
+def attn_window_pool(q, k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, sink, scale: float, window: int,
+                     pool: int, out, max_qlen: int = 0) -> None:
+  """out [T, H dv] = softmax attention of each new token over the tokens at most window - 1 places back (window 0:
+  all), the pooled blocks that end at or before position - window (pool 0: none), and the per-head sink logit."""
+  _mix("attn_window_pool", _gpu(q))(q, k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, sink, float(scale),
+                                    int(window), int(pool), out, int(max_qlen) or int(q.shape[0]))
+
+
+def ssd_prep(P, x_off: int, dt_off: int, conv_w, conv_b, conv_state, state_slots, cu_q, A_log, dt_bias, H: int, dv: int,
+             xbc, v, decay) -> None:
+  """SSD inputs of a step: xbc [T, C] = silu(causal conv of P[:, x_off : +C] + conv_b) (x | B | C channels),
+  dt = softplus(P[:, dt_off : +H] + dt_bias), v [T, H dv] = dt * x, decay [T, H] = exp(-exp(A_log) dt); the
+  convolution state [slots, taps - 1, C] takes the step's last inputs."""
+  _mix("ssd_prep", _gpu(P))(P, int(x_off), int(dt_off), conv_w, conv_b, conv_state, state_slots, cu_q, A_log, dt_bias,
+                            int(H), int(dv), xbc, v, decay)
+
+
+def ssd_gate_norm(o, xbc, skip_d, P, z_off: int, w, groups: int, eps: float, out) -> None:
+  """out[:, :inner] = group_rms_norm((o + D[head] * x) * silu(P[:, z_off : +inner])) * w, in `groups` equal parts."""
+  _mix("ssd_gate_norm", _gpu(o))(o, xbc, skip_d, P, int(z_off), w, int(groups), float(eps), out)
+
+
+def polynorm_act(P, up_off: int, F: int, coef, eps: float, out) -> None:
+  """out[:, :F] = a N(z) + b N(z^2) + c N(z^3) + e, z = P[:, up_off : +F], N = division by the row's RMS, coef = (a, b, c, e)."""
+  _mix("polynorm_act", _gpu(P))(P, int(up_off), int(F), coef, float(eps), out)
+
+
+def relu2(P, off: int, F: int, out) -> None:
+  """out[:, :F] = relu(P[:, off : +F])^2."""
+  _mix("relu2", _gpu(P))(P, int(off), int(F), out)
+
+
+def moe_weighted_sum(y, slot_of, topw, k: int, sh_y, P, shg_off: int, out) -> None:
+  """out [T, D] fp32 = sum_j topw[t, j] * y[slot_of[t, j]] (+ sigmoid(P[t, shg_off]) * sh_y[t] for a shared expert)."""
+  _mix("moe_weighted_sum", _gpu(y))(y, slot_of, topw, int(k), sh_y, P, int(shg_off), out)

@@ -333,6 +333,9 @@ def linear_recurrence(q, k, v, decay, beta, q_scale, state, state_slots, cu_q, o
         S *= decay[t].reshape(H, 1, 1)
         u = beta[t].reshape(H, 1) * (vt - torch.einsum("hdv,hd->hv", S, kt))
         S += kt[:, :, None] * u[:, None, :]
+      elif decay.numel() == decay.shape[0] * H:  # one decay per head
+        S *= decay[t].reshape(H, 1, 1)
+        S += kt[:, :, None] * vt[:, None, :]
       else:
         S *= decay[t].reshape(H, d, 1)
         S += kt[:, :, None] * vt[:, None, :]
@@ -346,3 +349,153 @@ def gated_rmsnorm(o, w, P, g_off, eps, out_scale, out):
   gate = P[:, g_off:g_off + x.shape[1] * dv].float().reshape(T, -1, dv)
   y = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float() * F.silu(gate) * out_scale
   out.copy_(y.reshape(T, -1).to(out.dtype))
+
+
+# ------------------------------------------------------------------ post-norm blocks: window attention, SSD, feed-forwards
+# Torch twins of csrc/hybrid.hip.
+def gated_postnorm(x, y, P, g_off, gate_b, alpha, w, eps, out):
+  """x <- (alpha x + y * sigmoid(P[:, g_off : +D] + gate_b)) / rms * w in place (P None: no gate); out[:, :D] = x."""
+  D = x.shape[1]
+  s = alpha * x
+  if y is not None:
+    yy = y[:, :D].float()
+    if P is not None:
+      yy = yy * torch.sigmoid(P[:, g_off:g_off + D].float() + gate_b.float())
+    s = s + yy
+  x.copy_(s / torch.sqrt(s.pow(2).mean(-1, keepdim=True) + eps) * w.float())
+  if out is not None:
+    out[:, :D] = x.to(out.dtype)
+
+
+def pool_dims(pool: int):
+  """(pooled entries per 64-token page, padded to whole 16-byte runs of the transposed value layout)."""
+  per = -(-PAGE // pool)
+  return per, -(-per // 8) * 8
+
+
+def qk_norm_rope_store(P, bias, q_off, k_off, v_off, H, G, d, dv, R, pos, cos_sin, slots, eps, qk_norm, q_out, k_cache,
+                       v_cache):
+  T = P.shape[0]
+  Pb = P.float() if bias is None else P.float() + bias.float()
+  half = R // 2
+
+  def prep(x):
+    if R:
+      cs = cos_sin[pos.long()]
+      c, s = cs[:, None, :half], cs[:, None, half:]
+      a, b = x[..., :half], x[..., half:R]
+      x = torch.cat([a * c - b * s, b * c + a * s, x[..., R:]], -1)
+    if qk_norm:
+      x = x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    return x
+  q_out.copy_(prep(Pb[:, q_off:q_off + H * d].reshape(T, H, d)).to(q_out.dtype))
+  if k_off < 0:
+    return
+  ok = slots >= 0
+  s = slots[ok].long()
+  k_cache[s // PAGE, :, s % PAGE] = prep(Pb[:, k_off:k_off + G * d].reshape(T, G, d))[ok].to(k_cache.dtype)
+  v_cache[s // PAGE, :, :, s % PAGE] = Pb[:, v_off:v_off + G * dv].reshape(T, G, dv)[ok].to(v_cache.dtype)
+
+
+def _pool_slot(blk: int, pool: int):
+  """Pooled block blk lives with the page that holds its last token: (page index in the sequence, entry)."""
+  pg = (blk * pool + pool - 1) // PAGE
+  return pg, blk - (pg * PAGE) // pool
+
+
+def kv_pool_update(k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, pool, max_qlen=0):
+  """Mean key / value of every block of `pool` tokens whose last token arrived in this step -> the pooled caches
+  kp [pages, G, per, d], vp [pages, G, dv, per8]."""
+  for b in range(ctx_lens.numel()):
+    n, q = int(ctx_lens[b]), int(cu_q[b + 1]) - int(cu_q[b])
+    if n <= 0 or q <= 0:
+      continue
+    for blk in range((n - q) // pool, (n - pool) // pool + 1):
+      toks = torch.arange(blk * pool, blk * pool + pool)
+      pages = block_tables[b, toks // PAGE].long()
+      pg, e = _pool_slot(blk, pool)
+      dst = int(block_tables[b, pg])
+      kp[dst, :, e] = k_cache[pages, :, toks % PAGE].float().mean(0).to(kp.dtype)
+      vp[dst, :, :, e] = v_cache[pages, :, :, toks % PAGE].float().mean(0).to(vp.dtype)
+
+
+def attn_window_pool(q, k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, sink, scale, window, pool, out, max_qlen=0):
+  T, H, d = q.shape
+  G, dv = k_cache.shape[1], v_cache.shape[2]
+  rep = H // G
+  for b in range(ctx_lens.numel()):
+    t0, t1, n = int(cu_q[b]), int(cu_q[b + 1]), int(ctx_lens[b])
+    if n <= 0 or t1 == t0:
+      continue
+    npg = -(-n // PAGE)
+    pages = block_tables[b, :npg].long()
+    k = k_cache[pages].permute(0, 2, 1, 3).reshape(npg * PAGE, G, d)[:n].float()
+    v = v_cache[pages].permute(0, 3, 1, 2).reshape(npg * PAGE, G, dv)[:n].float()
+    nb = n // pool if (pool and window) else 0
+    if nb:
+      loc = [_pool_slot(j, pool) for j in range(nb)]
+      pk = torch.stack([kp[int(block_tables[b, pg]), :, e].float() for pg, e in loc])  # [nb, G, d]
+      pv = torch.stack([vp[int(block_tables[b, pg]), :, :, e].float() for pg, e in loc])
+      k, v = torch.cat([k, pk]), torch.cat([v, pv])
+    qpos = torch.arange(n - (t1 - t0), n)[:, None]
+    kpos = torch.arange(n)[None, :]
+    vis = kpos <= qpos
+    if window:
+      vis = vis & (qpos - kpos < window)
+    if nb:
+      last = torch.arange(nb)[None, :] * pool + pool - 1
+      vis = torch.cat([vis, last <= qpos - window], 1)
+    s = torch.einsum("shd,thd->hst", q[t0:t1].float(), k.repeat_interleave(rep, 1)) * scale
+    s = s.masked_fill(~vis[None], float("-inf"))
+    if sink is not None:
+      s = torch.cat([s, sink.float()[:, None, None].expand(H, t1 - t0, 1)], -1)
+    w = torch.softmax(s, -1)[..., :k.shape[0]]
+    o = torch.einsum("hst,thd->shd", w, v.repeat_interleave(rep, 1))
+    out[t0:t1] = o.reshape(t1 - t0, H * dv).to(out.dtype)
+
+
+def ssd_prep(P, x_off, dt_off, conv_w, conv_b, conv_state, state_slots, cu_q, A_log, dt_bias, H, dv, xbc, v, decay):
+  C, taps = conv_w.shape
+  for b in range(state_slots.numel()):
+    t0, t1, slot = int(cu_q[b]), int(cu_q[b + 1]), int(state_slots[b])
+    if slot < 0 or t1 == t0:
+      continue
+    x = torch.cat([conv_state[slot], P[t0:t1, x_off:x_off + C].float()], 0)
+    y = F.silu(sum(conv_w[:, j].float() * x[j:j + t1 - t0] for j in range(taps)) + conv_b.float())
+    xbc[t0:t1] = y
+    if taps > 1:
+      conv_state[slot] = x[x.shape[0] - (taps - 1):]
+    dt = F.softplus(P[t0:t1, dt_off:dt_off + H].float() + dt_bias.float())
+    decay[t0:t1] = torch.exp(-torch.exp(A_log.float()) * dt)
+    v[t0:t1] = (y[:, :H * dv].reshape(-1, H, dv) * dt[:, :, None]).reshape(-1, H * dv)
+
+
+def ssd_gate_norm(o, xbc, skip_d, P, z_off, w, groups, eps, out):
+  T, inner = o.shape
+  H = skip_d.numel()
+  y = o.float() + (xbc[:, :inner].float().reshape(T, H, -1) * skip_d.float()[None, :, None]).reshape(T, inner)
+  y = (y * F.silu(P[:, z_off:z_off + inner].float())).reshape(T, groups, -1)
+  y = y / torch.sqrt(y.pow(2).mean(-1, keepdim=True) + eps)
+  out[:, :inner] = (y.reshape(T, inner) * w.float()).to(out.dtype)
+
+
+def polynorm_act(P, up_off, Fd, coef, eps, out):
+  z = P[:, up_off:up_off + Fd].float()
+  a, b, c, e = coef.float().tolist()
+
+  def nrm(t):
+    return t / torch.sqrt(t.pow(2).mean(-1, keepdim=True) + eps)
+  out[:, :Fd] = (a * nrm(z) + b * nrm(z * z) + c * nrm(z * z * z) + e).to(out.dtype)
+
+
+def relu2(P, off, Fd, out):
+  out[:, :Fd] = torch.relu(P[:, off:off + Fd].float()).pow(2).to(out.dtype)
+
+
+def moe_weighted_sum(y, slot_of, topw, k, sh_y, P, shg_off, out):
+  """out [T, D] = sum_j topw[t, j] y[slot_of[t, j]] (+ sigmoid(P[t, shg_off]) sh_y[t])."""
+  T, D = out.shape
+  acc = (y[slot_of.long().reshape(T, k), :D].float() * topw.reshape(T, k, 1)).sum(1)
+  if sh_y is not None:
+    acc = acc + torch.sigmoid(P[:, shg_off:shg_off + 1].float()) * sh_y[:, :D].float()
+  out.copy_(acc)

@@ -135,6 +135,8 @@ class ShardRunner:
     if use_graphs is None:
       # MoE routing runs on the device too (moe_route + grouped GEMMs), so every model is capturable
       use_graphs = self.device.type == "cuda" and os.environ.get("XOT_GRAPHS", "1") == "1"
+      if dtype == torch.float32 and config.is_mixed and any(s.ffn is not None and s.ffn.experts for s in config.layer_specs):
+        use_graphs = False  # an all-fp32 run groups the experts' rows on the host (vendor SGEMM per expert)
     self.use_graphs = use_graphs
     self._graphs: Dict[tuple, dict] = {}
     # decode graphs per (batch bucket, block-table width class): a step whose longest context fits a narrower
