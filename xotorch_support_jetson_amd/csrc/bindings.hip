@@ -7,6 +7,7 @@
 
 namespace xot {
 void bind_mixers(pybind11::module& m);  // csrc/mixers.hip
+void bind_hybrid(pybind11::module& m);  // csrc/hybrid.hip
 }
 
 namespace {
@@ -1019,6 +1020,7 @@ void adamw(at::Tensor& p, const at::Tensor& g, at::Tensor& m, at::Tensor& v, con
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "xot MI355X (gfx950) kernel library";
   xot::bind_mixers(m);
+  xot::bind_hybrid(m);
   m.def("rmsnorm", &rmsnorm);
   m.def("rmsnorm_bwd", &rmsnorm_bwd, py::arg("x"), py::arg("w"), py::arg("dy"), py::arg("dx"), py::arg("dw"),
         py::arg("eps"), py::arg("res") = py::none());

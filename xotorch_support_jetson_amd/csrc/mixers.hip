@@ -15,45 +15,11 @@
 //
 // A fused projection's output P is fp32 [T, ldp]; "column offset" arguments address its slices.  Activations that
 // feed the next GEMM (AT) are bf16 or fp32; everything that enters a norm, a score or a recurrence is fp32.
-#include <torch/extension.h>
-#include <ATen/hip/HIPContext.h>
-#include "common.h"
+#include "mixer_util.h"
 
 namespace xot {
 namespace {
-
-constexpr int PAGE_TOK = 64;
-
-__device__ __forceinline__ float ldf(const float* p) { return *p; }
-__device__ __forceinline__ float ldf(const uint16_t* p) { return bf2f(*p); }
-__device__ __forceinline__ void stf(float* p, float v) { *p = v; }
-__device__ __forceinline__ void stf(uint16_t* p, float v) { *p = f2bf(v); }
-
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
-__device__ __forceinline__ float siluf_(float x) { return x / (1.0f + expf(-x)); }
-__device__ __forceinline__ float softplusf_(float x) { return log1pf(expf(-fabsf(x))) + fmaxf(x, 0.0f); }
-__device__ __forceinline__ float logsigmoidf_(float x) { return fminf(x, 0.0f) - log1pf(expf(-fabsf(x))); }
-
-__device__ __forceinline__ float block_sum(float v, float* red) {
-  v = wave_sum(v);
-  const int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[w] = v;
-  __syncthreads();
-  float t = 0.0f;
-  for (int i = 0; i < nw; ++i) t += red[i];
-  return t;
-}
-
-// sequence of token t: the b with cu[b] <= t < cu[b + 1]
-__device__ __forceinline__ int seq_of(const int* cu, int B, int t) {
-  int lo = 0, hi = B - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (cu[mid] <= t) lo = mid; else hi = mid - 1;
-  }
-  return lo;
-}
+using namespace mix;
 
 // ------------------------------------------------------------------ residual + scalar-gain RMS norm
 template <typename AT>
@@ -139,16 +105,6 @@ __global__ void rope_kv_store_k(const float* __restrict__ P, int ldp, int q_off,
 // Wave-per-(token, head) kernel (any d <= 256, bf16 or fp32; the fallback for more than 8 query heads per kv head):
 // lanes over keys for the scores, then lanes over value dims for the weighted sum.
 constexpr int ATT_TILE = 512;
-
-__device__ __forceinline__ void ld8(const float* p, float* o) {
-  const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
-  o[0] = a[0]; o[1] = a[1]; o[2] = a[2]; o[3] = a[3]; o[4] = b[0]; o[5] = b[1]; o[6] = b[2]; o[7] = b[3];
-}
-__device__ __forceinline__ void ld8(const uint16_t* p, float* o) {
-  const s16x8 a = ld16(p);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) o[i] = bf2f(a[i]);
-}
 
 template <typename AT>
 __global__ void attn_gated_chunk_k(const AT* __restrict__ q, const AT* __restrict__ k_cache, const AT* __restrict__ v_cache,
@@ -598,7 +554,9 @@ __global__ void gla_prep_k(const float* __restrict__ P, int ldp, int a1_off, int
 // contiguous runs and a token's k / q slices are vector LDS reads.  The launcher uses RS = 16 (a whole DPP row per
 // value channel).  Tokens are staged through LDS TB at a time, double-buffered: the next block's global loads are in flight
 // while the current one is consumed.
-// DELTA: S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q.   else: S = diag(a) S + k v^T; o = S^T q.
+// MODE 1 (delta rule): S *= g; u = beta (v - S^T k); S += k u^T; o = S^T q.   MODE 0: S = diag(a) S + k v^T; o = S^T q
+// (a decay per key channel).   MODE 2: S = g S + k v^T; o = S^T q (one decay per head: the state-space-duality form
+// with k = B, q = C, v = dt x).
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
   const int m = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false);
@@ -615,17 +573,18 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
-template <int KR, int RS, bool DELTA>
+template <int KR, int RS, int MODE>
 __global__ __launch_bounds__(256) void linear_recurrence_k(
     const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk, const float* __restrict__ v, int ldv,
     const float* __restrict__ decay, const float* __restrict__ beta, float q_scale, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_q, int H, int G, int d, int dv,
     float* __restrict__ out) {
   constexpr int DP = KR * RS;  // padded key dim
+  constexpr bool DELTA = MODE == 1, SCALAR = MODE != 0;
   constexpr int COLS = 256 / RS;
   constexpr int TB = DP >= 256 ? 8 : 16;
   constexpr int NQ = TB * DP / 256, NV = (TB * COLS + 255) / 256;
-  __shared__ __attribute__((aligned(16))) float sq[2][TB][DP], sk[2][TB][DP], sa[2][TB][DELTA ? 4 : DP];
+  __shared__ __attribute__((aligned(16))) float sq[2][TB][DP], sk[2][TB][DP], sa[2][TB][SCALAR ? 4 : DP];
   __shared__ float sv[2][TB][COLS], sg[2][TB][2];
   const int b = blockIdx.x, h = blockIdx.y, cb = blockIdx.z;
   const int slot = state_slots[b];
@@ -653,7 +612,7 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
     }
   }
 
-  float pq[NQ], pk[NQ], pa[DELTA ? 1 : NQ], pv[NV], pg0 = 0.0f, pg1 = 0.0f;
+  float pq[NQ], pk[NQ], pa[SCALAR ? 1 : NQ], pv[NV], pg0 = 0.0f, pg1 = 0.0f;
   auto fetch = [&](int tb) {  // global -> registers: tokens tb .. tb + TB - 1 of the sequence (zeros past its end)
 #pragma unroll
     for (int j = 0; j < NQ; ++j) {
@@ -662,16 +621,16 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
       const bool in = i < d && tb + tt < n;
       pq[j] = in ? q[t * ldq + hk * d + i] * q_scale : 0.0f;
       pk[j] = in ? k[t * ldk + hk * d + i] : 0.0f;
-      if (!DELTA) pa[j] = in ? decay[(t * H + h) * d + i] : 0.0f;
+      if (!SCALAR) pa[j] = in ? decay[(t * H + h) * d + i] : 0.0f;
     }
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int e = tid + 256 * j, tt = e / COLS, c = cb * COLS + e % COLS;
       pv[j] = (e < TB * COLS && c < dv && tb + tt < n) ? v[(int64_t)(t0 + tb + tt) * ldv + h * dv + c] : 0.0f;
     }
-    if (DELTA && tid < TB && tb + tid < n) {
+    if (SCALAR && tid < TB && tb + tid < n) {
       pg0 = decay[(int64_t)(t0 + tb + tid) * H + h];
-      pg1 = beta[(int64_t)(t0 + tb + tid) * H + h];
+      if (DELTA) pg1 = beta[(int64_t)(t0 + tb + tid) * H + h];
     }
   };
   auto stage = [&](int buf) {  // registers -> LDS
@@ -680,14 +639,14 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
       const int e = tid + 256 * j, tt = e / DP, i = e - tt * DP;
       sq[buf][tt][i] = pq[j];
       sk[buf][tt][i] = pk[j];
-      if (!DELTA) sa[buf][tt][i] = pa[j];
+      if (!SCALAR) sa[buf][tt][i] = pa[j];
     }
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int e = tid + 256 * j;
       if (e < TB * COLS) sv[buf][e / COLS][e % COLS] = pv[j];
     }
-    if (DELTA && tid < TB) {
+    if (SCALAR && tid < TB) {
       sg[buf][tid][0] = pg0;
       sg[buf][tid][1] = pg1;
     }
@@ -723,6 +682,14 @@ __global__ __launch_bounds__(256) void linear_recurrence_k(
 #pragma unroll
         for (int m = 0; m < KR; ++m) {
           s[m] += kk[m] * u;
+          const float p = s[m] * qq[m];
+          if ((m & 3) == 0) o0 += p; else if ((m & 3) == 1) o1 += p; else if ((m & 3) == 2) o2 += p; else o3 += p;
+        }
+      } else if (SCALAR) {
+        const float g = sg[buf][tt][0];
+#pragma unroll
+        for (int m = 0; m < KR; ++m) {
+          s[m] = g * s[m] + kk[m] * vc;
           const float p = s[m] * qq[m];
           if ((m & 3) == 0) o0 += p; else if ((m & 3) == 1) o1 += p; else if ((m & 3) == 2) o2 += p; else o3 += p;
         }
@@ -771,31 +738,6 @@ __global__ void gated_rmsnorm_k(const float* __restrict__ o, const float* __rest
 }
 
 // ------------------------------------------------------------------ host side
-#define MCHECK(cond, ...) TORCH_CHECK(cond, "xot mixers: ", __VA_ARGS__)
-
-inline hipStream_t stream() { return at::hip::getCurrentHIPStream().stream(); }
-inline bool is_act(const at::Tensor& t) { return t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kFloat; }
-inline void f32c(const at::Tensor& t, const char* name) {
-  MCHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), name, " must be a contiguous fp32 GPU tensor");
-}
-inline void i32c(const at::Tensor& t, const char* name) {
-  MCHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), name, " must be a contiguous int32 GPU tensor");
-}
-// fused projection output: fp32 rows of unit inner stride
-inline int ld_of(const at::Tensor& P, const char* name) {
-  MCHECK(P.is_cuda() && P.scalar_type() == at::kFloat && P.dim() == 2 && P.stride(1) == 1, name, " must be fp32 [T, n] rows");
-  return (int)P.stride(0);
-}
-inline void cols_ok(const at::Tensor& P, int64_t off, int64_t n, const char* what) {
-  MCHECK(off >= 0 && n >= 0 && off + n <= P.size(1), what, ": columns [", off, ", ", off + n, ") outside the projection");
-}
-// activation output rows (bf16 / fp32), maybe a column slice of a wider buffer
-inline int act_ld(const at::Tensor& t, int64_t T, int64_t n, const char* name) {
-  MCHECK(t.is_cuda() && is_act(t) && t.dim() == 2 && t.size(0) == T && t.size(1) == n && t.stride(1) == 1, name,
-         " must be [T, ", n, "] bf16 / fp32 rows");
-  return (int)t.stride(0);
-}
-
 void resid_scale_norm(at::Tensor& x, const c10::optional<at::Tensor>& y1, const c10::optional<at::Tensor>& s1,
                       const c10::optional<at::Tensor>& y2, const c10::optional<at::Tensor>& s2,
                       const c10::optional<at::Tensor>& gain, double eps, const c10::optional<at::Tensor>& out) {
@@ -1044,13 +986,13 @@ void gla_prep(const at::Tensor& P, int64_t a1_off, const at::Tensor& a2, const a
                                                          decay.data_ptr<float>());
 }
 
-template <int RS, bool DELTA>
+template <int RS, int MODE>
 void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* decay,
                 const float* beta, float q_scale, float* state, const int* slots, const int* cu, int H, int G, int d, int dv,
                 float* out) {
 #define REC_CASE(DPAD)                                                                                                 \
   case DPAD:                                                                                                           \
-    linear_recurrence_k<DPAD / RS, RS, DELTA><<<grid, 256, 0, stream()>>>(q, ldq, k, ldk, v, ldv, decay, beta, q_scale, \
+    linear_recurrence_k<DPAD / RS, RS, MODE><<<grid, 256, 0, stream()>>>(q, ldq, k, ldk, v, ldv, decay, beta, q_scale, \
                                                                           state, slots, cu, H, G, d, dv, out);         \
     break;
   switch (KR * RS) {  // padded key dim
@@ -1065,8 +1007,9 @@ void launch_rec(int KR, dim3 grid, const float* q, int ldq, const float* k, int 
 #undef REC_CASE
 }
 
-// q / k [T, G d], v [T, H dv]: fp32 rows of unit inner stride (column slices allowed).  decay [T, H] (delta) or
-// [T, H d] (per key channel); beta [T, H] (delta only).  state [slots, H, dv, d] (S^T: key rows contiguous).
+// q / k [T, G d], v [T, H dv]: fp32 rows of unit inner stride (column slices allowed).  decay [T, H] (delta rule, or
+// without beta: one decay per head and a plain outer-product write) or [T, H d] (per key channel); beta [T, H] (delta
+// only).  state [slots, H, dv, d] (S^T: key rows contiguous).
 void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& decay,
                        const c10::optional<at::Tensor>& beta, double q_scale, at::Tensor& state, const at::Tensor& state_slots,
                        const at::Tensor& cu_q, at::Tensor& out) {
@@ -1088,9 +1031,10 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   if (delta) {
     f32c(*beta, "beta");
     MCHECK(beta->numel() == T * H && decay.numel() == T * H, "delta rule: beta / decay must be [T, H]");
-  } else {
+  } else if (decay.numel() != T * H) {
     MCHECK(decay.numel() == T * H * d && G == H, "per-channel decay must be [T, H d] with one q / k head per value head");
   }
+  const bool scalar = !delta && decay.numel() == T * H;  // one decay per head, q / k shared by H / G heads
   int DP = 16;
   while (DP < d) DP *= 2;
   MCHECK(DP <= 256, "linear_recurrence: key dim above 256");
@@ -1104,7 +1048,7 @@ void linear_recurrence(const at::Tensor& q, const at::Tensor& k, const at::Tenso
   launch_rec<R, D>(DP / R, grid, q.data_ptr<float>(), ldq, k.data_ptr<float>(), ldk, v.data_ptr<float>(), ldv,              \
                    decay.data_ptr<float>(), bp, (float)q_scale, state.data_ptr<float>(), state_slots.data_ptr<int>(),        \
                    cu_q.data_ptr<int>(), (int)H, (int)G, (int)d, (int)dv, out.data_ptr<float>())
-  if (delta) REC_GO(16, true); else REC_GO(16, false);
+  if (delta) REC_GO(16, 1); else if (scalar) REC_GO(16, 2); else REC_GO(16, 0);
 #undef REC_GO
 }
 

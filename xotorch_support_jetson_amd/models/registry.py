@@ -66,6 +66,7 @@ _CARDS: List[tuple] = [
   ("tiny-deepseek-v3", 3, "synthetic/tiny-deepseek-v3", "Tiny DeepSeek-V3 (synthetic)"),
   ("tiny-llava", 4, "synthetic/tiny-llava", "Tiny LLaVA (synthetic)"),
   ("tiny-tarepel", 4, "synthetic/tiny-tarepel", "Tiny Tarepel (synthetic)"),
+  ("tiny-mogelix", 4, "synthetic/tiny-mogelix", "Tiny Mogelix (synthetic)"),
 ]
 
 model_cards: Dict[str, dict] = {mid: {"layers": n, "repo": {ENGINE: repo}} for mid, n, repo, _ in _CARDS}

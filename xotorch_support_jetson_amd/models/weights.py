@@ -334,11 +334,13 @@ def prepare_for_decode(sw: "ShardWeights", keep_rowmajor: Iterable[str] = (), fp
     return out
 
   if sw.config.is_mixed:  # fused projections of mixed-layer models (bf16 runs; an fp32 run keeps vendor SGEMM layouts)
+    def wide(t):  # (the tall-M tiles start at 128 output columns: narrower projections stay row-major)
+      return conv(t) if t is not None and t.shape[0] >= 128 else t
     for lw in sw.layers.values():
       if lw.in_w.dtype == torch.bfloat16:
-        lw.in_w, lw.out_w, lw.down_w, lw.ff_w = conv(lw.in_w), conv(lw.out_w), conv(lw.down_w), conv(lw.ff_w)
+        lw.in_w, lw.out_w, lw.down_w, lw.ff_w = wide(lw.in_w), wide(lw.out_w), wide(lw.down_w), wide(lw.ff_w)
     if sw.lm_head is not None and sw.lm_head.dtype == torch.bfloat16:
-      sw.lm_head = conv(sw.lm_head)
+      sw.lm_head = wide(sw.lm_head)
     return sw
 
   proj = conv8 if fp8 else conv
