@@ -77,7 +77,8 @@ def _batch(lens_done, lens_new, pages, dev, scramble):
 ATTN = [  # H, G, d, dv, R, window, pool, sink
   (4, 2, 32, 32, 16, 24, 6, True), (2, 2, 64, 64, 64, 70, 11, True), (3, 1, 16, 48, 0, 0, 0, True),
   (2, 1, 128, 32, 32, 7, 1, False), (16, 1, 16, 16, 8, 20, 64, True), (6, 2, 20, 12, 4, 33, 5, True),
-  (2, 1, 96, 160, 32, 50, 0, False), (2, 2, 256, 256, 64, 70, 7, True), (4, 4, 64, 64, 64, 1, 2, True)]
+  (2, 1, 96, 160, 32, 50, 0, False), (2, 2, 256, 256, 64, 70, 7, True), (4, 4, 64, 64, 64, 1, 2, True),
+  (2, 1, 128, 128, 64, 40, 9, True), (4, 2, 64, 64, 32, 0, 0, False), (2, 2, 32, 32, 0, 100, 3, False)]
 
 
 @pytest.mark.parametrize("dev,dtype", DEVS)
@@ -107,9 +108,9 @@ def test_window_attention_with_pooled_blocks(dev, dtype, H, G, d, dv, R, window,
   vc = torch.zeros(pages, G, dv, 64, dtype=adt, device=dev)
   kp = vp = None
   if window and pool:
-    per, per8 = K.pool_dims(pool)
-    kp = torch.full((pages, G, per, d), float("nan"), dtype=adt, device=dev)  # an entry read before it is written shows
-    vp = torch.full((pages, G, dv, per8), float("nan"), dtype=adt, device=dev)
+    per = K.pool_dims(pool)
+    kp = torch.full((pages, G, per, d), 1e4, dtype=adt, device=dev)  # an entry read before it is written shows
+    vp = torch.full((pages, G, per, dv), 1e4, dtype=adt, device=dev)
   W = torch.cat([t["q"], t["k"], t["v"]], 0)
   bias = torch.cat([t["q.b"], t["k.b"], t["v.b"]]).float().to(dev)
   sc = rot and dict(rope_type="llama3", factor=4.0, low_freq_factor=1.0, high_freq_factor=4.0,
@@ -151,9 +152,9 @@ def test_single_tokens_read_the_same_caches(dev, dtype):
   pages = 4
   kc = torch.zeros(pages, G, 64, d, dtype=dtype, device=dev)
   vc = torch.zeros(pages, G, dv, 64, dtype=dtype, device=dev)
-  per, per8 = K.pool_dims(pool)
+  per = K.pool_dims(pool)
   kp = torch.zeros(pages, G, per, d, dtype=dtype, device=dev)
-  vp = torch.zeros(pages, G, dv, per8, dtype=dtype, device=dev)
+  vp = torch.zeros(pages, G, per, dv, dtype=dtype, device=dev)
   W = torch.cat([t["q"], t["k"], t["v"]], 0)
   bias = torch.cat([t["q.b"], t["k.b"], t["v.b"]]).float().to(dev)
   tab = torch.zeros(1, 0, device=dev)

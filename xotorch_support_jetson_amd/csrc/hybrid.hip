@@ -110,13 +110,13 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_k(
 
 // ------------------------------------------------------------------ pooled keys and values
 // Block j holds the positions j pool .. j pool + pool - 1; its mean key / value is stored with the page of its last
-// token, entry j - floor(64 page / pool): kp [pages, G, per, d], vp [pages, G, dv, per8].  Workgroup = (completed
+// token, entry j - floor(64 page / pool): kp [pages, G, per, d], vp [pages, G, per, dv].  Workgroup = (completed
 // block of the step, sequence, kv head); the means are taken over the caches' contents as they hold them.
 template <typename AT>
 __global__ void kv_pool_update_k(const AT* __restrict__ k_cache, const AT* __restrict__ v_cache, AT* __restrict__ kp,
                                  AT* __restrict__ vp, const int* __restrict__ block_tables, int width,
-                                 const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int pool, int per, int per8,
-                                 int G, int d, int dv) {
+                                 const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, int pool, int per, int G,
+                                 int d, int dv) {
   const int b = blockIdx.y, g = blockIdx.z;
   const int ctx = ctx_lens[b], nq = cu_q[b + 1] - cu_q[b];
   if (ctx <= 0 || nq <= 0) return;
@@ -138,7 +138,7 @@ __global__ void kv_pool_update_k(const AT* __restrict__ k_cache, const AT* __res
       const int iv = i - d;
       for (int p = first; p <= lastp; ++p)
         acc += ldf(v_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * dv + iv) * PAGE_TOK + (p % PAGE_TOK));
-      stf(vp + (dst * dv + iv) * per8 + e, acc / np);
+      stf(vp + (dst * per + e) * dv + iv, acc / np);
     }
   }
 }
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(64) void attn_window_pool_k(
     const AT* __restrict__ q, const AT* __restrict__ k_cache, const AT* __restrict__ v_cache, const AT* __restrict__ kp,
     const AT* __restrict__ vp, const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_lens, int B, const float* __restrict__ sink, float scale, int window, int pool, int per,
-    int per8, AT* __restrict__ out, int ldo, int H, int G, int d, int dv) {
+    AT* __restrict__ out, int ldo, int H, int G, int d, int dv) {
   extern __shared__ float sm[];
   float* qs = sm;      // [d]
   float* ws = sm + d;  // [WATT_TILE]
@@ -225,11 +225,11 @@ __global__ __launch_bounds__(64) void attn_window_pool_k(
     for (int j = a0; j < a0 + n; ++j) {
       const float w = ws[j - a0];
       const int pgi = (j * pool + pool - 1) / PAGE_TOK;
-      const AT* vr = vp + ((int64_t)bt[pgi] * G + g) * dv * per8 + (j - (pgi * PAGE_TOK) / pool);
+      const AT* vr = vp + (((int64_t)bt[pgi] * G + g) * per + (j - (pgi * PAGE_TOK) / pool)) * dv;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const int i = lane + 64 * c;
-        if (i < dv) acc[c] += w * ldf(vr + (int64_t)i * per8);
+        if (i < dv) acc[c] += w * ldf(vr + i);
       }
     }
   }
@@ -261,6 +261,214 @@ __global__ __launch_bounds__(64) void attn_window_pool_k(
   for (int c = 0; c < 4; ++c) {
     const int i = lane + 64 * c;
     if (i < dv) stf(out + (int64_t)t * ldo + h * dv + i, acc[c] * inv);
+  }
+}
+
+// MFMA kernel (bf16, d = dv = 32 NK): a workgroup owns 128 consecutive queries of one (sequence, head), 32 per wave, and
+// walks first the pooled blocks that its last query sees, then the tokens from its first query's window on, a tile of
+// KT keys at a time: the K rows and V^T runs of the tile are staged in LDS and shared by the four waves (pooled
+// entries are gathered row by row and their values transposed on the way in).  Scores are computed transposed,
+// S^T = K Q^T (keys x queries), so a lane's accumulator rows are consecutive keys of ONE query: the running maximum and
+// denominator are per lane (the four lanes of a query agree on the maximum through two shuffles and keep partial
+// denominators), and the exponentials, rounded to bf16, are as they lie the B operand of O^T += V^T P^T, whose k slots
+// (g, j) are read as keys {4g .. 4g+3, 16+4g .. 16+4g+3} on both operands.  Scores, maxima and sums are fp32 (base-2
+// exponentials of scores scaled by log2 e); the sink's logit starts the running maximum with a denominator of one.
+template <int NK>
+__global__ __launch_bounds__(256) void attn_window_pool_mfma_k(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache,
+    const uint16_t* __restrict__ kp, const uint16_t* __restrict__ vp, const int* __restrict__ block_tables, int width,
+    const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, const float* __restrict__ sink, float scale, int window,
+    int pool, int per, uint16_t* __restrict__ out, int ldo, int H, int G) {
+  constexpr int D = NK * 32, ND = NK * 2, QT = 2;
+  constexpr int KT = D > 192 ? 32 : 64;  // keys per tile (a page holds a whole number of tiles)
+  constexpr int KP = D + 8, VP = KT + 8;
+  constexpr float L2E = 1.4426950408889634f;
+  __shared__ __attribute__((aligned(16))) uint16_t sK[KT][KP], sV[D][VP];
+  const int b = blockIdx.x, h = blockIdx.z;
+  const int wave = threadIdx.x >> 6, l = threadIdx.x & 63, c = l & 15, g4 = l >> 4;
+  const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0, ctx = ctx_lens[b];
+  const int wq0 = blockIdx.y * 128;
+  if (ctx <= 0 || wq0 >= qlen) return;
+  const int q0 = wq0 + wave * 32;
+  const bool active = q0 < qlen;
+  const int nq = active ? min(32, qlen - q0) : 0;
+  const int pos0 = ctx - qlen + q0;  // position of the wave's first query
+  const int gk = h / (H / G);
+  // pooled blocks a query at position p sees: those that end at or before p - window
+  auto blocks_seen = [&](int p) { return (pool > 0 && p - window + 1 >= pool) ? (p - window + 1) / pool : 0; };
+  s16x8 qf[QT][NK];
+  int qpos[QT], qnb[QT];
+  float m[QT], lsum[QT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int local = qt * 16 + c;
+    const bool ok = local < nq;
+    qpos[qt] = pos0 + local;
+    qnb[qt] = blocks_seen(qpos[qt]);
+    const uint16_t* qp = q + ((int64_t)(t0 + q0 + local) * H + h) * D + 8 * g4;
+#pragma unroll
+    for (int ks = 0; ks < NK; ++ks) qf[qt][ks] = ok ? ld16(qp + ks * 32) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    m[qt] = sink ? sink[h] * L2E : -INFINITY;
+    lsum[qt] = (sink && g4 == 0) ? 1.0f : 0.0f;  // (partial denominators: one of the query's four lanes counts the sink)
+  }
+  f32x4 o[QT][ND];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+    for (int db = 0; db < ND; ++db) o[qt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float sc2 = scale * L2E;
+  const int* bt = block_tables + (int64_t)b * width;
+  const int wlast = ctx - qlen + wq0 + min(128, qlen - wq0) - 1;  // the workgroup's last query
+  const int wpos0 = ctx - qlen + wq0;
+  const int last = active ? pos0 + nq - 1 : -1;                  // the wave's last query
+  constexpr int NCHUNK = KT * (D / 8), NCH = (NCHUNK + 255) / 256;
+  s16x8 rk[NCH], rv[NCH];
+
+  // one staged tile: scores, mask, running softmax, O^T += V^T P^T.  pooled: key index = block index.
+  auto consume = [&](int tb, bool pooled) {
+#pragma unroll
+    for (int sub = 0; sub < KT / 32; ++sub) {
+      const int kb = tb + sub * 32;
+      bool full;
+      if (pooled) {
+        if (!active || kb >= blocks_seen(last)) continue;  // (wave-uniform) none of these blocks is seen by this wave
+        full = kb + 32 <= blocks_seen(pos0);
+      } else {
+        const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+        if (!active || kb > last || kb + 31 < k_lo) continue;
+        full = kb + 31 <= pos0 && (window <= 0 || kb > last - window);
+      }
+      f32x4 s[2][QT];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) s[kt][qt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+          const s16x8 a = ld16(&sK[sub * 32 + kt * 16 + c][ks * 32 + 8 * g4]);
+#pragma unroll
+          for (int qt = 0; qt < QT; ++qt) s[kt][qt] = mfma16(a, qf[qt][ks], s[kt][qt]);
+        }
+      s16x8 pf[QT];
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float t = s[kt][qt][r] * sc2;
+            if (!full) {
+              const int kpos = kb + kt * 16 + 4 * g4 + r;
+              const bool vis = pooled ? kpos < qnb[qt] : (kpos <= qpos[qt] && (window <= 0 || qpos[qt] - kpos < window));
+              t = vis ? t : -INFINITY;
+            }
+            s[kt][qt][r] = t;
+            mx = fmaxf(mx, t);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(m[qt], mx);
+        const float ms = mn == -INFINITY ? 0.0f : mn;  // (nothing seen yet: every weight below is exp2(-inf) = 0)
+        const float corr = __builtin_amdgcn_exp2f(m[qt] - ms);
+        m[qt] = mn;
+        float ps = 0.0f;
+        u32x4 packed;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int r2 = 0; r2 < 2; ++r2) {
+            const float p0 = __builtin_amdgcn_exp2f(s[kt][qt][2 * r2] - ms), p1 = __builtin_amdgcn_exp2f(s[kt][qt][2 * r2 + 1] - ms);
+            ps += p0 + p1;
+            // two bf16 (rounded half up: the weights are in [0, 1]) in one dword
+            packed[kt * 2 + r2] = __builtin_amdgcn_perm(__float_as_uint(p1) + 0x8000u, __float_as_uint(p0) + 0x8000u, 0x07060302u);
+          }
+        pf[qt] = __builtin_bit_cast(s16x8, packed);
+        lsum[qt] = lsum[qt] * corr + ps;
+#pragma unroll
+        for (int db = 0; db < ND; ++db) o[qt][db] *= corr;
+      }
+      // (slots no token has written yet hold zeros or an earlier request's finite values; their weight is 0)
+#pragma unroll
+      for (int db = 0; db < ND; ++db) {
+        const s16x4 v0 = *reinterpret_cast<const s16x4*>(&sV[db * 16 + c][sub * 32 + 4 * g4]);
+        const s16x4 v1 = *reinterpret_cast<const s16x4*>(&sV[db * 16 + c][sub * 32 + 16 + 4 * g4]);
+        const s16x8 a = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) o[qt][db] = mfma16(a, pf[qt], o[qt][db]);
+      }
+    }
+  };
+
+  // ---- pooled blocks [0, nbw): rows gathered from the pages that hold them, values transposed into sV
+  const int nbw = blocks_seen(wlast);
+  for (int tb = 0; tb < nbw; tb += KT) {
+    __syncthreads();  // the previous tile has been consumed
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int ch = threadIdx.x + 256 * j;
+      if (NCHUNK % 256 != 0 && ch >= NCHUNK) break;
+      const int row = ch / (D / 8), cc = ch - row * (D / 8);
+      const int blk = min(tb + row, nbw - 1);  // (rows past the last block repeat it; their weight is 0)
+      const int pgi = (blk * pool + pool - 1) / PAGE_TOK;
+      const int64_t e = ((int64_t)bt[pgi] * G + gk) * per + (blk - (pgi * PAGE_TOK) / pool);
+      st16(&sK[row][cc * 8], ld16(kp + e * D + cc * 8));
+      const s16x8 v = ld16(vp + e * D + cc * 8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sV[cc * 8 + i][row] = (uint16_t)v[i];
+    }
+    __syncthreads();
+    consume(tb, true);
+  }
+
+  // ---- tokens from the first query's window on
+  const int t_lo = (window > 0 ? max(0, wpos0 - window + 1) : 0) & ~(KT - 1);
+  auto fetch = [&](int tb) {
+    const int64_t pg = (int64_t)bt[tb >> 6] * G + gk;
+    const int koff = tb & 63;
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int ch = threadIdx.x + 256 * j;
+      if (NCHUNK % 256 != 0 && ch >= NCHUNK) break;
+      const int row = ch / (D / 8), cc = ch - row * (D / 8);
+      rk[j] = ld16(k_cache + ((pg * PAGE_TOK) + koff + row) * D + cc * 8);
+      const int vrow = ch / (KT / 8), vc = ch - vrow * (KT / 8);
+      rv[j] = ld16(v_cache + (pg * D + vrow) * PAGE_TOK + koff + vc * 8);
+    }
+  };
+  fetch(t_lo);
+  for (int tb = t_lo; tb <= wlast; tb += KT) {
+    __syncthreads();  // the previous tile has been consumed
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const int ch = threadIdx.x + 256 * j;
+      if (NCHUNK % 256 != 0 && ch >= NCHUNK) break;
+      const int row = ch / (D / 8), cc = ch - row * (D / 8);
+      st16(&sK[row][cc * 8], rk[j]);
+      const int vrow = ch / (KT / 8), vc = ch - vrow * (KT / 8);
+      st16(&sV[vrow][vc * 8], rv[j]);
+    }
+    __syncthreads();
+    if (tb + KT <= wlast) fetch(tb + KT);  // in flight while this tile is consumed
+    consume(tb, false);
+  }
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    float ls = lsum[qt];
+    ls += __shfl_xor(ls, 16, 64);
+    ls += __shfl_xor(ls, 32, 64);
+    if (qt * 16 + c >= nq) continue;
+    const float inv = ls > 0.0f ? 1.0f / ls : 0.0f;
+    uint16_t* op = out + (int64_t)(t0 + q0 + qt * 16 + c) * ldo + h * D + 4 * g4;
+#pragma unroll
+    for (int db = 0; db < ND; ++db) {
+      s16x4 w;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) w[r] = (short)f2bf(o[qt][db][r] * inv);
+      *reinterpret_cast<s16x4*>(op + db * 16) = w;
+    }
   }
 }
 
@@ -392,6 +600,9 @@ __global__ void moe_weighted_sum_k(const float* __restrict__ y, int ldy, const i
 }
 
 // ------------------------------------------------------------------ host side
+// XOT_WATT_MFMA=0 keeps prompt portions on the wave-per-token attention kernel (A/B runs)
+const bool WATT_MFMA = []() { const char* e = getenv("XOT_WATT_MFMA"); return !(e && e[0] == '0'); }();
+
 void gated_postnorm(at::Tensor& x, const c10::optional<at::Tensor>& y, const c10::optional<at::Tensor>& P, int64_t g_off,
                     const c10::optional<at::Tensor>& gate_b, double alpha, const at::Tensor& w, double eps,
                     const c10::optional<at::Tensor>& out) {
@@ -478,16 +689,15 @@ void qk_norm_rope_store(const at::Tensor& P, const c10::optional<at::Tensor>& bi
 }
 
 void check_pools(const at::Tensor& k_cache, const at::Tensor& kp, const at::Tensor& vp, int64_t pool, int64_t G, int64_t d,
-                 int64_t dv, int* per, int* per8) {
+                 int64_t dv, int* per) {
   MCHECK(pool >= 1, "pool must be at least one token");
   *per = (int)((PAGE_TOK + pool - 1) / pool);
-  *per8 = (*per + 7) / 8 * 8;
   MCHECK(kp.is_cuda() && kp.scalar_type() == k_cache.scalar_type() && kp.is_contiguous() && kp.dim() == 4 &&
              kp.size(0) == k_cache.size(0) && kp.size(1) == G && kp.size(2) == *per && kp.size(3) == d,
          "the pooled keys must be [pages, G, ceil(64 / pool), d] of the caches' dtype");
   MCHECK(vp.is_cuda() && vp.scalar_type() == k_cache.scalar_type() && vp.is_contiguous() && vp.dim() == 4 &&
-             vp.size(0) == k_cache.size(0) && vp.size(1) == G && vp.size(2) == dv && vp.size(3) == *per8,
-         "the pooled values must be [pages, G, dv, ceil(64 / pool) rounded up to 8] of the caches' dtype");
+             vp.size(0) == k_cache.size(0) && vp.size(1) == G && vp.size(2) == *per && vp.size(3) == dv,
+         "the pooled values must be [pages, G, ceil(64 / pool), dv] of the caches' dtype");
 }
 
 void kv_pool_update(const at::Tensor& k_cache, const at::Tensor& v_cache, at::Tensor& kp, at::Tensor& vp,
@@ -496,8 +706,8 @@ void kv_pool_update(const at::Tensor& k_cache, const at::Tensor& v_cache, at::Te
   MCHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && is_act(k_cache), "caches must be 4-D bf16 / fp32");
   const int64_t G = k_cache.size(1), d = k_cache.size(3), dv = v_cache.size(2), B = ctx_lens.numel();
   check_kv(k_cache, v_cache, k_cache.scalar_type(), G, d, dv);
-  int per, per8;
-  check_pools(k_cache, kp, vp, pool, G, d, dv, &per, &per8);
+  int per;
+  check_pools(k_cache, kp, vp, pool, G, d, dv, &per);
   i32c(block_tables, "block_tables");
   i32c(cu_q, "cu_q");
   i32c(ctx_lens, "ctx_lens");
@@ -509,15 +719,26 @@ void kv_pool_update(const at::Tensor& k_cache, const at::Tensor& v_cache, at::Te
     kv_pool_update_k<uint16_t><<<grid, bs, 0, stream()>>>(
         (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(), (uint16_t*)kp.data_ptr(),
         (uint16_t*)vp.data_ptr(), block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(),
-        ctx_lens.data_ptr<int>(), (int)pool, per, per8, (int)G, (int)d, (int)dv);
+        ctx_lens.data_ptr<int>(), (int)pool, per, (int)G, (int)d, (int)dv);
   else
     kv_pool_update_k<float><<<grid, bs, 0, stream()>>>(
         k_cache.data_ptr<float>(), v_cache.data_ptr<float>(), kp.data_ptr<float>(), vp.data_ptr<float>(),
         block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)pool,
-        per, per8, (int)G, (int)d, (int)dv);
+        per, (int)G, (int)d, (int)dv);
 }
 
-// max_qlen: the longest run of new tokens of one sequence in this step.
+template <int NK>
+void launch_wattn_mfma(dim3 grid, const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache, const uint16_t* kp,
+                       const uint16_t* vp, const at::Tensor& block_tables, const at::Tensor& cu_q, const at::Tensor& ctx_lens,
+                       const float* sink, float scale, int window, int pool, int per, at::Tensor& out, int ldo, int H, int G) {
+  attn_window_pool_mfma_k<NK><<<grid, 256, 0, stream()>>>(
+      (const uint16_t*)q.data_ptr(), (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(), kp, vp,
+      block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), sink, scale,
+      window, pool, per, (uint16_t*)out.data_ptr(), ldo, H, G);
+}
+
+// max_qlen: the longest run of new tokens of one sequence in this step (below 16: single decoded tokens and short
+// portions -> the wave-per-token kernel; the MFMA kernel takes bf16 with d == dv in {32, 64, 128}).
 void attn_window_pool(const at::Tensor& q, const at::Tensor& k_cache, const at::Tensor& v_cache,
                       const c10::optional<at::Tensor>& kp, const c10::optional<at::Tensor>& vp, const at::Tensor& block_tables,
                       const at::Tensor& cu_q, const at::Tensor& ctx_lens, const c10::optional<at::Tensor>& sink, double scale,
@@ -530,11 +751,11 @@ void attn_window_pool(const at::Tensor& q, const at::Tensor& k_cache, const at::
   check_kv(k_cache, v_cache, q.scalar_type(), G, d, dv);
   MCHECK(G > 0 && H % G == 0 && d <= 256 && dv <= 256, "head counts / sizes (at most 256)");
   MCHECK(window >= 0 && pool >= 0, "window / pool must not be negative");
-  int per = 0, per8 = 0;
+  int per = 0;
   const bool pooled = pool > 0 && window > 0;
   if (pooled) {
     MCHECK(kp.has_value() && vp.has_value(), "pooled blocks need the pooled caches");
-    check_pools(k_cache, *kp, *vp, pool, G, d, dv, &per, &per8);
+    check_pools(k_cache, *kp, *vp, pool, G, d, dv, &per);
   }
   i32c(block_tables, "block_tables");
   i32c(cu_q, "cu_q");
@@ -548,6 +769,23 @@ void attn_window_pool(const at::Tensor& q, const at::Tensor& k_cache, const at::
   }
   MCHECK(out.scalar_type() == q.scalar_type(), "out must have q's dtype");
   const int ldo = act_ld(out, T, H * dv, "out");
+  if (q.scalar_type() == at::kBFloat16 && max_qlen >= 16 && d == dv && (d == 32 || d == 64 || d == 128) && ldo % 4 == 0 &&
+      WATT_MFMA) {
+    const dim3 grid((unsigned)B, (unsigned)((max_qlen + 127) / 128), (unsigned)H);
+    const uint16_t* kpp = pooled ? (const uint16_t*)kp->data_ptr() : nullptr;
+    const uint16_t* vpp = pooled ? (const uint16_t*)vp->data_ptr() : nullptr;
+    const int pl = pooled ? (int)pool : 0;
+    if (d == 32)
+      launch_wattn_mfma<1>(grid, q, k_cache, v_cache, kpp, vpp, block_tables, cu_q, ctx_lens, sp, (float)scale, (int)window, pl,
+                           per, out, ldo, (int)H, (int)G);
+    else if (d == 64)
+      launch_wattn_mfma<2>(grid, q, k_cache, v_cache, kpp, vpp, block_tables, cu_q, ctx_lens, sp, (float)scale, (int)window, pl,
+                           per, out, ldo, (int)H, (int)G);
+    else
+      launch_wattn_mfma<4>(grid, q, k_cache, v_cache, kpp, vpp, block_tables, cu_q, ctx_lens, sp, (float)scale, (int)window, pl,
+                           per, out, ldo, (int)H, (int)G);
+    return;
+  }
   const dim3 grid((unsigned)T, (unsigned)H);
   const size_t lds = (size_t)(d + WATT_TILE) * sizeof(float);
   if (q.scalar_type() == at::kBFloat16)
@@ -555,14 +793,14 @@ void attn_window_pool(const at::Tensor& q, const at::Tensor& k_cache, const at::
         (const uint16_t*)q.data_ptr(), (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(),
         pooled ? (const uint16_t*)kp->data_ptr() : nullptr, pooled ? (const uint16_t*)vp->data_ptr() : nullptr,
         block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, sp,
-        (float)scale, (int)window, pooled ? (int)pool : 0, per, per8, (uint16_t*)out.data_ptr(), ldo, (int)H, (int)G, (int)d,
+        (float)scale, (int)window, pooled ? (int)pool : 0, per, (uint16_t*)out.data_ptr(), ldo, (int)H, (int)G, (int)d,
         (int)dv);
   else
     attn_window_pool_k<float><<<grid, 64, lds, stream()>>>(
         q.data_ptr<float>(), k_cache.data_ptr<float>(), v_cache.data_ptr<float>(),
         pooled ? kp->data_ptr<float>() : nullptr, pooled ? vp->data_ptr<float>() : nullptr, block_tables.data_ptr<int>(),
         (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, sp, (float)scale, (int)window,
-        pooled ? (int)pool : 0, per, per8, out.data_ptr<float>(), ldo, (int)H, (int)G, (int)d, (int)dv);
+        pooled ? (int)pool : 0, per, out.data_ptr<float>(), ldo, (int)H, (int)G, (int)d, (int)dv);
 }
 
 void ssd_prep(const at::Tensor& P, int64_t x_off, int64_t dt_off, const at::Tensor& conv_w, const at::Tensor& conv_b,

@@ -102,7 +102,7 @@ class KVCache:
       self.k = [None if a is None else torch.zeros(num_pages, a[0], PAGE, a[1], device=device, dtype=dtype) for a in dims]
       self.v = [None if a is None else torch.zeros(num_pages, a[0], a[2], PAGE, device=device, dtype=dtype) for a in dims]
       # window attention with pooled blocks: per layer the (source layer, block size) pooled caches it reads, K
-      # [pages, G, per, d] and V [pages, G, dv, per8]; entries live with the page of a block's last token, so they are
+      # [pages, G, per, d] and V [pages, G, per, dv]; entries live with the page of a block's last token, so they are
       # handed out and returned with the sequence's pages.  pool_owner[j]: this layer fills them (the first layer of
       # the shard that reads this source with this block size); a layer that borrows another's keys and values aliases
       # that layer's pools.
@@ -121,9 +121,9 @@ class KVCache:
         self.k[j], self.v[j] = self.k[js], self.v[js]
         if a.pool > 0 and a.window > 0:
           if (src, a.pool) not in made:
-            per, per8 = K.pool_dims(a.pool)
+            per = K.pool_dims(a.pool)
             made[(src, a.pool)] = (torch.zeros(num_pages, a.kv_heads, per, a.dim, device=device, dtype=dtype),
-                                   torch.zeros(num_pages, a.kv_heads, a.vdim, per8, device=device, dtype=dtype))
+                                   torch.zeros(num_pages, a.kv_heads, per, a.vdim, device=device, dtype=dtype))
             self.pool_owner[j] = True
           self.kp[j], self.vp[j] = made[(src, a.pool)]
       return
@@ -145,8 +145,7 @@ class KVCache:
           n += a[0] * PAGE * (a[1] + a[2]) * itemsize
         if w is not None and w.pool > 0 and w.window > 0 and (w.kv_from if w.kv_from >= 0 else i, w.pool) not in seen:
           seen.add((w.kv_from if w.kv_from >= 0 else i, w.pool))
-          per, per8 = K.pool_dims(w.pool)
-          n += w.kv_heads * (per * w.dim + per8 * w.vdim) * itemsize
+          n += w.kv_heads * K.pool_dims(w.pool) * (w.dim + w.vdim) * itemsize
       return max(1, n)
     if c.is_mla:
       return n_layers * PAGE * c.mla_dim * 2

@@ -520,7 +520,7 @@ def qk_norm_rope_store(P, bias, q_off: int, k_off: int, v_off: int, H: int, G: i
 
 def kv_pool_update(k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, pool: int, max_qlen: int) -> None:
   """Mean key and value of every block of `pool` consecutive tokens whose last token is among the step's new ones,
-  read from the paged caches as they hold them, into the pooled caches kp [pages, G, per, d] / vp [pages, G, dv, per8]
+  read from the paged caches as they hold them, into the pooled caches kp [pages, G, per, d] / vp [pages, G, per, dv]
   (entry of block b: with the page of its last token, see pool_dims)."""
   _mix("kv_pool_update", _gpu(k_cache))(k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, int(pool), int(max_qlen))
 

@@ -367,10 +367,9 @@ def gated_postnorm(x, y, P, g_off, gate_b, alpha, w, eps, out):
     out[:, :D] = x.to(out.dtype)
 
 
-def pool_dims(pool: int):
-  """(pooled entries per 64-token page, padded to whole 16-byte runs of the transposed value layout)."""
-  per = -(-PAGE // pool)
-  return per, -(-per // 8) * 8
+def pool_dims(pool: int) -> int:
+  """Pooled entries per 64-token page: the most blocks of `pool` tokens whose last token lies in one page."""
+  return -(-PAGE // pool)
 
 
 def qk_norm_rope_store(P, bias, q_off, k_off, v_off, H, G, d, dv, R, pos, cos_sin, slots, eps, qk_norm, q_out, k_cache,
@@ -405,7 +404,7 @@ def _pool_slot(blk: int, pool: int):
 
 def kv_pool_update(k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, pool, max_qlen=0):
   """Mean key / value of every block of `pool` tokens whose last token arrived in this step -> the pooled caches
-  kp [pages, G, per, d], vp [pages, G, dv, per8]."""
+  kp [pages, G, per, d], vp [pages, G, per, dv]."""
   for b in range(ctx_lens.numel()):
     n, q = int(ctx_lens[b]), int(cu_q[b + 1]) - int(cu_q[b])
     if n <= 0 or q <= 0:
@@ -416,7 +415,7 @@ def kv_pool_update(k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, pool,
       pg, e = _pool_slot(blk, pool)
       dst = int(block_tables[b, pg])
       kp[dst, :, e] = k_cache[pages, :, toks % PAGE].float().mean(0).to(kp.dtype)
-      vp[dst, :, :, e] = v_cache[pages, :, :, toks % PAGE].float().mean(0).to(vp.dtype)
+      vp[dst, :, e] = v_cache[pages, :, :, toks % PAGE].float().mean(0).to(vp.dtype)
 
 
 def attn_window_pool(q, k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, sink, scale, window, pool, out, max_qlen=0):
@@ -435,7 +434,7 @@ def attn_window_pool(q, k_cache, v_cache, kp, vp, block_tables, cu_q, ctx_lens, 
     if nb:
       loc = [_pool_slot(j, pool) for j in range(nb)]
       pk = torch.stack([kp[int(block_tables[b, pg]), :, e].float() for pg, e in loc])  # [nb, G, d]
-      pv = torch.stack([vp[int(block_tables[b, pg]), :, :, e].float() for pg, e in loc])
+      pv = torch.stack([vp[int(block_tables[b, pg]), :, e].float() for pg, e in loc])
       k, v = torch.cat([k, pk]), torch.cat([v, pv])
     qpos = torch.arange(n - (t1 - t0), n)[:, None]
     kpos = torch.arange(n)[None, :]
