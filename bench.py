@@ -135,20 +135,41 @@ def mixer_configs(name: str):
   return mixed, dense
 
 
-def bench_mixers(args):
-  """Prefill and decode throughput of Tarepel-design layers at sizes like a real model's (random weights), beside
-  the closest existing model (a Llama-style stack of equal width, depth, heads and feed-forward) on the same
-  runner: one prefill step of --mixer-batch prompts of --prompt-len tokens, then HIP-graph decode steps at that
-  context.  One JSON line; not the headline metric."""
+def hybrid_configs(name: str):
+  """(Mogelix-design config, the closest existing model: the Tarepel-design stack of equal width and depth).  Window
+  attention (the Tarepel chunk as window, pooled blocks of 64 tokens, sink) with a PolyNorm feed-forward alternates
+  with a Mamba-2 mixer (inner width 2 x width, state 128) under a relu^2 mixture of 8 experts, 2 chosen, plus a shared
+  expert."""
+  from xotorch_support_jetson_amd.models.config import from_hf_config
+  z = MIXER_SIZES[name]
+  H, G, d, chunk, rot = z["attn"]
+  W = z["width"]
+  att = {"type": "attention", "mlp": {"kind": "dense", "ff": z["ff"]},
+         "mixer": {"heads": H, "kv_heads": G, "dim": d, "vdim": d, "mask": {"size": chunk, "pool": 64}, "scale": d ** -0.5,
+                   "rot": {"base": 1e6, "dims": rot, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
+  ssd = {"type": "mamba2", "mixer": {"heads": 2 * W // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8},
+         "mlp": {"kind": "moe", "expert": {"ff": (z["ff"] // 2 + 127) // 128 * 128}, "router": {"experts": 8, "top": 2},
+                 "shared": {"ff": 1024}}}
+  hybrid = from_hf_config({"architecture": "Mogelix", "vocab": 32000, "width": W, "norm": {"eps": 1e-5}, "postln_alpha": 2.0,
+                           "layers": [att if i % 2 == 0 else ssd for i in range(z["layers"])]})
+  return hybrid, mixer_configs(name)[0]
+
+
+def bench_mixers(args, sizes=None, kinds=("tarepel", "llama"), configs=mixer_configs,
+                 what="Tarepel-design layers beside a Llama-style stack of equal size"):
+  """Prefill and decode throughput of mixed-layer designs at sizes like a real model's (random weights), beside
+  the closest existing model (--mixers: Tarepel beside a Llama-style stack of equal width, depth, heads and
+  feed-forward; --hybrid: Mogelix beside Tarepel) on the same runner: one prefill step of --mixer-batch prompts of
+  --prompt-len tokens, then HIP-graph decode steps at that context.  One JSON line; not the headline metric."""
   from xotorch_support_jetson_amd.inference.shard import Shard
   from xotorch_support_jetson_amd.runtime.runner import ShardRunner
   dev = torch.device("cuda:0")
   torch.cuda.set_device(dev)
   B, L = args.mixer_batch, args.prompt_len
   res = {}
-  for name in args.mixers.split(","):
+  for name in (sizes or args.mixers).split(","):
     row = {}
-    for kind, cfg in zip(("tarepel", "llama"), mixer_configs(name)):
+    for kind, cfg in zip(kinds, configs(name)):
       shard = Shard(f"{kind}-{name}", 0, cfg.num_layers - 1, cfg.num_layers)
       max_ctx = L + args.warmup + args.steps + 8
       r = ShardRunner(cfg, shard, dev, num_pages=B * -(-max_ctx // 64) + 4, max_batch=B, max_ctx=max_ctx, seed=0)
@@ -176,11 +197,11 @@ def bench_mixers(args):
       row[kind] = {"params_m": round(cfg.num_params() / 1e6, 1), "prefill_tok_s": round(B * L / t_pre, 1),
                    "prefill_ms": round(t_pre * 1e3, 2), "decode_tok_s": round(B / t_dec, 1),
                    "decode_ms_per_step": round(t_dec * 1e3, 3)}
-      log(f"[mixers {name}] {kind}: {row[kind]}")
+      log(f"[{name}] {kind}: {row[kind]}")
       del r
       torch.cuda.empty_cache()
     res[name] = row
-  print(json.dumps({"metric": "prefill / decode tokens/sec of Tarepel-design layers beside a Llama-style stack of equal size",
+  print(json.dumps({"metric": "prefill / decode tokens/sec of " + what,
                     "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": "bf16",
                     "data": "synthetic prompts, random-init weights", "batch": B, "prompt_len": L, "sizes": res}), flush=True)
 
@@ -208,11 +229,17 @@ def main():
   ap.add_argument("--mixers", default=None, metavar="SIZES",
                   help="instead of the headline: Tarepel-design layers beside a Llama-style stack at the named sizes "
                        f"(comma-separated, of {', '.join(MIXER_SIZES)}); one GPU")
-  ap.add_argument("--mixer-batch", type=int, default=16, help="--mixers: sequences per step")
+  ap.add_argument("--hybrid", default=None, metavar="SIZES",
+                  help="instead of the headline: Mogelix-design layers (window attention with pooled blocks, Mamba-2, "
+                       "relu^2 experts) beside the Tarepel-design stack at the named sizes; one GPU")
+  ap.add_argument("--mixer-batch", type=int, default=16, help="--mixers / --hybrid: sequences per step")
   args = ap.parse_args()
   os.environ["XOT_WEIGHT_DTYPE"] = args.weight_dtype
   if args.mixers:
     return bench_mixers(args)
+  if args.hybrid:
+    return bench_mixers(args, args.hybrid, ("mogelix", "tarepel"), hybrid_configs,
+                        "Mogelix-design layers beside a Tarepel-design stack of equal size")
 
   from xotorch_support_jetson_amd.models.config import preset
   from xotorch_support_jetson_amd.parallel.comm import P2PTransport, init_distributed

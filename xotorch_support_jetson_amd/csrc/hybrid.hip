@@ -4,7 +4,7 @@
 //   gated_postnorm      x <- rms_norm(alpha x + y * sigmoid(gate + b)) * w, and its copy in the GEMM operand dtype
 //   qk_norm_rope_store  q / k / v biases, partial rotate-half RoPE, per-head RMS division, paged write of k and v
 //   kv_pool_update      mean key / value of every block of `pool` tokens that the step completed -> pooled caches
-//   attn_window_pool    softmax attention over [window tokens | pooled blocks before the window | sink]: a wave per
+//   attn_window_pool    softmax attention over [window tokens | pooled blocks before the window | sink]: a workgroup per
 //                       (token, head) for any sizes and fp32; an MFMA kernel for bf16 prompt portions
 //   ssd_prep            causal convolution + bias + SiLU over x | B | C, dt = softplus(dt + bias), decay, v = dt x
 //   ssd_gate_norm       (o + D x) * silu(z), RMS norm in equal groups, weight
@@ -147,29 +147,34 @@ __global__ void kv_pool_update_k(const AT* __restrict__ k_cache, const AT* __res
 // A query at position i sees the tokens j with 0 <= i - j < window (window 0: all j <= i) and the pooled blocks b with
 // b pool + pool - 1 <= i - window; the softmax's denominator also holds exp(sink[head]).
 //
-// Wave per (token, head) (any d, dv <= 256, bf16 or fp32): the running maximum starts at the sink's logit with a
-// denominator of one; keys are walked a tile at a time, lanes over keys for the scores, then lanes over value dims for
-// the weighted sum (token values 8 keys per 16-byte V^T load).
+// Workgroup per (token, head) (any d, dv <= 256, bf16 or fp32), WATT_WAVES waves: the key tiles are dealt to the waves
+// in turn; a wave's running maximum starts at -inf (wave 0: at the sink's logit with a denominator of one), lanes go
+// over keys for the scores, then over value dims for the weighted sum (token values 8 keys per 16-byte V^T load); at
+// the end the waves' (maximum, denominator, sums) are merged through LDS.
 constexpr int WATT_TILE = 256;
+constexpr int WATT_WAVES = 8;
 
 template <typename AT>
-__global__ __launch_bounds__(64) void attn_window_pool_k(
+__global__ __launch_bounds__(64 * WATT_WAVES) void attn_window_pool_k(
     const AT* __restrict__ q, const AT* __restrict__ k_cache, const AT* __restrict__ v_cache, const AT* __restrict__ kp,
     const AT* __restrict__ vp, const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_lens, int B, const float* __restrict__ sink, float scale, int window, int pool, int per,
     AT* __restrict__ out, int ldo, int H, int G, int d, int dv) {
   extern __shared__ float sm[];
-  float* qs = sm;      // [d]
-  float* ws = sm + d;  // [WATT_TILE]
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float* qs = sm;                                     // [d]
+  float* ws = sm + d + wave * WATT_TILE;              // [WATT_TILE] per wave
+  float* mg = sm + d + WATT_WAVES * WATT_TILE;        // merge: [waves][2 + dv]
+  const int t = blockIdx.x, h = blockIdx.y;
   const int b = seq_of(cu_q, B, t);
   const int ctx = ctx_lens[b];
   if (ctx <= 0) return;  // padding row of a captured decode batch
   const int pos = ctx - (cu_q[b + 1] - cu_q[b]) + (t - cu_q[b]);
   const int g = h / (H / G);
-  for (int i = lane; i < d; i += 64) qs[i] = ldf(q + ((int64_t)t * H + h) * d + i);
+  for (int i = threadIdx.x; i < d; i += blockDim.x) qs[i] = ldf(q + ((int64_t)t * H + h) * d + i);
+  __syncthreads();
   const int* bt = block_tables + (int64_t)b * width;
-  float m = sink ? sink[h] : -INFINITY, l = sink ? 1.0f : 0.0f;
+  float m = (sink && wave == 0) ? sink[h] : -INFINITY, l = (sink && wave == 0) ? 1.0f : 0.0f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};  // value dims lane, lane + 64, ...
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int nbv = (pool > 0 && window > 0 && pos - window + 1 >= pool) ? (pos - window + 1) / pool : 0;
@@ -188,10 +193,12 @@ __global__ __launch_bounds__(64) void attn_window_pool_k(
     }
     return s * scale;
   };
-  // one tile: scores of the keys a0 + [0, n) (those outside [p0, p1) weigh nothing) -> softmax weights in ws, the
-  // running maximum / denominator / accumulators rescaled
+  // one tile of this wave: scores of the keys a0 + [0, n) (those outside [p0, p1) weigh nothing) -> softmax weights in
+  // ws, the running maximum / denominator / accumulators rescaled.  ws is the wave's own: its lanes' LDS accesses
+  // are ordered by the wave-level fences.
   auto weigh = [&](int a0, int n, int p0, int p1, auto&& key_row) {
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
     float mx = -INFINITY;
     for (int p = a0 + lane; p < a0 + n; p += 64) {
       float s = -INFINITY;
@@ -212,11 +219,14 @@ __global__ __launch_bounds__(64) void attn_window_pool_k(
 #pragma unroll
     for (int c = 0; c < 4; ++c) acc[c] *= corr;
     m = mn;
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
   };
 
+  int tile = 0;  // tiles are dealt to the waves in turn
   // pooled blocks [0, nbv)
-  for (int a0 = 0; a0 < nbv; a0 += WATT_TILE) {
+  for (int a0 = 0; a0 < nbv; a0 += WATT_TILE, ++tile) {
+    if (tile % WATT_WAVES != wave) continue;
     const int n = min(WATT_TILE, nbv - a0);
     weigh(a0, n, 0, nbv, [&](int j) {
       const int pgi = (j * pool + pool - 1) / PAGE_TOK;
@@ -234,7 +244,8 @@ __global__ __launch_bounds__(64) void attn_window_pool_k(
     }
   }
   // tokens [lo, pos], tiles aligned to 8 keys
-  for (int a0 = lo & ~7; a0 <= pos; a0 += WATT_TILE) {
+  for (int a0 = lo & ~7; a0 <= pos; a0 += WATT_TILE, ++tile) {
+    if (tile % WATT_WAVES != wave) continue;
     const int a1 = min(a0 + WATT_TILE, (pos + 8) & ~7);
     weigh(a0, a1 - a0, lo, pos + 1, [&](int p) {
       return k_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * PAGE_TOK + (p % PAGE_TOK)) * d;
@@ -256,11 +267,33 @@ __global__ __launch_bounds__(64) void attn_window_pool_k(
       }
     }
   }
-  const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+  // merge the waves: M = max m_w, out = sum_w acc_w e^(m_w - M) / sum_w l_w e^(m_w - M)
+  float* mine = mg + wave * (2 + dv);
+  if (lane == 0) {
+    mine[0] = m;
+    mine[1] = l;
+  }
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     const int i = lane + 64 * c;
-    if (i < dv) stf(out + (int64_t)t * ldo + h * dv + i, acc[c] * inv);
+    if (i < dv) mine[2 + i] = acc[c];
+  }
+  __syncthreads();
+  float M = -INFINITY;
+  for (int w = 0; w < WATT_WAVES; ++w) M = fmaxf(M, mg[w * (2 + dv)]);
+  float L = 0.0f;
+  for (int w = 0; w < WATT_WAVES; ++w) {
+    const float mw = mg[w * (2 + dv)];
+    if (mw != -INFINITY) L += mg[w * (2 + dv) + 1] * expf(mw - M);
+  }
+  const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+  for (int i = threadIdx.x; i < dv; i += blockDim.x) {
+    float a = 0.0f;
+    for (int w = 0; w < WATT_WAVES; ++w) {
+      const float mw = mg[w * (2 + dv)];
+      if (mw != -INFINITY) a += mg[w * (2 + dv) + 2 + i] * expf(mw - M);
+    }
+    stf(out + (int64_t)t * ldo + h * dv + i, a * inv);
   }
 }
 
@@ -490,7 +523,7 @@ __global__ void ssd_prep_k(const float* __restrict__ P, int ldp, int x_off, int 
   const float* row = P + (int64_t)t * ldp;
   const float* st = conv_state + (int64_t)slot * (taps - 1) * C;
   const int inner = H * dv;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
     float acc = conv_b[c];
     for (int j = 0; j < taps; ++j) {
       const int sidx = local - (taps - 1 - j);
@@ -504,8 +537,9 @@ __global__ void ssd_prep_k(const float* __restrict__ P, int ldp, int x_off, int 
       v[(int64_t)t * inner + c] = softplusf_(row[dt_off + h] + dt_bias[h]) * y;
     }
   }
-  for (int h = threadIdx.x; h < H; h += blockDim.x)
-    decay[(int64_t)t * H + h] = expf(-expf(A_log[h]) * softplusf_(row[dt_off + h] + dt_bias[h]));
+  if (blockIdx.y == 0)
+    for (int h = threadIdx.x; h < H; h += blockDim.x)
+      decay[(int64_t)t * H + h] = expf(-expf(A_log[h]) * softplusf_(row[dt_off + h] + dt_bias[h]));
 }
 
 // the last taps - 1 convolution inputs of every sequence -> its state slot (after every token of the step has read
@@ -586,14 +620,21 @@ __global__ void relu2_k(const float* __restrict__ P, int ldp, int off, int F, AT
 }
 
 // ------------------------------------------------------------------ routed experts' weighted sum + gated shared expert
+// y [splits * slots, >= D]: the down projection's K slices (summed here in a fixed order)
 __global__ void moe_weighted_sum_k(const float* __restrict__ y, int ldy, const int* __restrict__ slot_of,
-                                   const float* __restrict__ topw, int k, const float* __restrict__ sh, int lds,
-                                   const float* __restrict__ P, int ldp, int shg_off, float* __restrict__ out, int D) {
+                                   const float* __restrict__ topw, int k, int splits, int64_t slots,
+                                   const float* __restrict__ sh, int lds, const float* __restrict__ P, int ldp, int shg_off,
+                                   float* __restrict__ out, int D) {
   const int64_t t = blockIdx.x;
   const float sg = sh ? sigmoidf_(P[t * ldp + shg_off]) : 0.0f;
   for (int i = threadIdx.x; i < D; i += blockDim.x) {
     float acc = 0.0f;
-    for (int j = 0; j < k; ++j) acc += topw[t * k + j] * y[(int64_t)slot_of[t * k + j] * ldy + i];
+    for (int j = 0; j < k; ++j) {
+      const int64_t r = slot_of[t * k + j];
+      float ys = 0.0f;
+      for (int sp = 0; sp < splits; ++sp) ys += y[(sp * slots + r) * ldy + i];
+      acc += topw[t * k + j] * ys;
+    }
     if (sh) acc += sg * sh[t * lds + i];
     out[t * D + i] = acc;
   }
@@ -787,16 +828,16 @@ void attn_window_pool(const at::Tensor& q, const at::Tensor& k_cache, const at::
     return;
   }
   const dim3 grid((unsigned)T, (unsigned)H);
-  const size_t lds = (size_t)(d + WATT_TILE) * sizeof(float);
+  const size_t lds = (size_t)(d + WATT_WAVES * WATT_TILE + WATT_WAVES * (2 + dv)) * sizeof(float);
   if (q.scalar_type() == at::kBFloat16)
-    attn_window_pool_k<uint16_t><<<grid, 64, lds, stream()>>>(
+    attn_window_pool_k<uint16_t><<<grid, 64 * WATT_WAVES, lds, stream()>>>(
         (const uint16_t*)q.data_ptr(), (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(),
         pooled ? (const uint16_t*)kp->data_ptr() : nullptr, pooled ? (const uint16_t*)vp->data_ptr() : nullptr,
         block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, sp,
         (float)scale, (int)window, pooled ? (int)pool : 0, per, (uint16_t*)out.data_ptr(), ldo, (int)H, (int)G, (int)d,
         (int)dv);
   else
-    attn_window_pool_k<float><<<grid, 64, lds, stream()>>>(
+    attn_window_pool_k<float><<<grid, 64 * WATT_WAVES, lds, stream()>>>(
         q.data_ptr<float>(), k_cache.data_ptr<float>(), v_cache.data_ptr<float>(),
         pooled ? kp->data_ptr<float>() : nullptr, pooled ? vp->data_ptr<float>() : nullptr, block_tables.data_ptr<int>(),
         (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, sp, (float)scale, (int)window,
@@ -828,7 +869,9 @@ void ssd_prep(const at::Tensor& P, int64_t x_off, int64_t dt_off, const at::Tens
   MCHECK(xbc.numel() == T * C && v.numel() == T * H * dv && decay.numel() == T * H, "ssd_prep: output shape mismatch");
   cols_ok(P, x_off, C, "conv inputs");
   cols_ok(P, dt_off, H, "dt");
-  ssd_prep_k<<<T, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)x_off, (int)dt_off, conv_w.data_ptr<float>(),
+  // few tokens (decode steps): the channels are spread over workgroups too
+  const dim3 pgrid((unsigned)T, (unsigned)(T >= 2048 ? 1 : std::min<int64_t>((C + 255) / 256, 32)));
+  ssd_prep_k<<<pgrid, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)x_off, (int)dt_off, conv_w.data_ptr<float>(),
                                       conv_b.data_ptr<float>(), (int)taps, (int)C, conv_state.data_ptr<float>(),
                                       state_slots.data_ptr<int>(), cu_q.data_ptr<int>(), (int)B, A_log.data_ptr<float>(),
                                       dt_bias.data_ptr<float>(), (int)H, (int)dv, xbc.data_ptr<float>(), v.data_ptr<float>(),
@@ -902,7 +945,7 @@ void relu2(const at::Tensor& P, int64_t off, int64_t F, at::Tensor& out) {
 
 void moe_weighted_sum(const at::Tensor& y, const at::Tensor& slot_of, const at::Tensor& topw, int64_t k,
                       const c10::optional<at::Tensor>& sh_y, const c10::optional<at::Tensor>& P, int64_t shg_off,
-                      at::Tensor& out) {
+                      at::Tensor& out, int64_t splits) {
   const int ldy = ld_of(y, "y");
   f32c(out, "out");
   f32c(topw, "topw");
@@ -910,7 +953,8 @@ void moe_weighted_sum(const at::Tensor& y, const at::Tensor& slot_of, const at::
   MCHECK(out.dim() == 2, "out must be [T, D]");
   const int64_t T = out.size(0), D = out.size(1);
   if (T == 0) return;
-  MCHECK(k >= 1 && topw.numel() == T * k && slot_of.numel() == T * k && y.size(0) == T * k && y.size(1) >= D,
+  MCHECK(k >= 1 && splits >= 1 && topw.numel() == T * k && slot_of.numel() == T * k && y.size(0) == splits * T * k &&
+             y.size(1) >= D,
          "moe_weighted_sum: shape mismatch");
   const float *sp = nullptr, *pp = nullptr;
   int lds = 0, ldp = 0;
@@ -925,12 +969,14 @@ void moe_weighted_sum(const at::Tensor& y, const at::Tensor& slot_of, const at::
   }
   // (slot_of comes from the routing kernel: every entry is a row of y)
   moe_weighted_sum_k<<<T, 256, 0, stream()>>>(y.data_ptr<float>(), ldy, slot_of.data_ptr<int>(), topw.data_ptr<float>(), (int)k,
-                                              sp, lds, pp, ldp, (int)shg_off, out.data_ptr<float>(), (int)D);
+                                              (int)splits, (int64_t)(T * k), sp, lds, pp, ldp, (int)shg_off,
+                                              out.data_ptr<float>(), (int)D);
 }
 
 }  // namespace
 
 void bind_hybrid(pybind11::module& m) {
+  namespace py = pybind11;
   m.def("gated_postnorm", &gated_postnorm);
   m.def("qk_norm_rope_store", &qk_norm_rope_store);
   m.def("kv_pool_update", &kv_pool_update);
@@ -939,7 +985,8 @@ void bind_hybrid(pybind11::module& m) {
   m.def("ssd_gate_norm", &ssd_gate_norm);
   m.def("polynorm_act", &polynorm_act);
   m.def("relu2", &relu2);
-  m.def("moe_weighted_sum", &moe_weighted_sum);
+  m.def("moe_weighted_sum", &moe_weighted_sum, py::arg("y"), py::arg("slot_of"), py::arg("topw"), py::arg("k"),
+        py::arg("sh_y"), py::arg("P"), py::arg("shg_off"), py::arg("out"), py::arg("splits") = 1);
 }
 
 }  // namespace xot

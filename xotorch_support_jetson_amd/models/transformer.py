@@ -583,15 +583,26 @@ class ShardModel:
       slot_of[order] = torch.arange(T * k)
       sorted_tok = (order // k).int()
       off = torch.cat([torch.zeros(1, dtype=torch.long), torch.bincount(topi.long(), minlength=E).cumsum(0)]).int()
-    Fp = lw.ex_up_w.shape[1]
+    Fp, Dq, S = lw.ex_up_w.shape[1], lw.ex_down_w.shape[1], 1
     if hn.dtype == torch.bfloat16 and hn.is_cuda:
+      # rows per expert decide the kernel as for the framework's other expert layers: the weight-streaming grouped GEMM
+      # for decode-sized groups (down projection split over K), gemm_big tiles once the groups are compute-bound
       C = require()
+      sh_up, sh_dn = layout_of(lw.ex_up_w) == "stream", layout_of(lw.ex_down_w) == "stream"
+      per_expert = T * k / E
+      big = sh_up and sh_dn and per_expert >= MOE_BIG_MIN_ROWS and Fp % 256 == 0 and Dq % 256 == 0
+      bm, bm_dn, S_dn = moe_tiles(per_expert, E) if big else (0, 0, 0)
+      if MOE_PP2:
+        bm, bm_dn = ({256: 2256, 192: 2192}.get(t, t) for t in (bm, bm_dn))
+      S = S_dn if big else (4 if T * k <= 64 else 2)
+      if Fp % (256 * S):
+        S = 1
       up = torch.empty(T * k, Fp, dtype=torch.float32, device=dev)
-      C.gemm_moe(hn, lw.ex_up_w, up, off, sorted_tok, K.EPI["none"], T, layout_of(lw.ex_up_w) == "stream", 1, 0)
+      C.gemm_moe(hn, lw.ex_up_w, up, off, sorted_tok, K.EPI["none"], T, sh_up, 1, bm)
       act = torch.empty(T * k, Fp, dtype=torch.bfloat16, device=dev)
       K.relu2(up, 0, Fp, act)
-      y = torch.empty(T * k, lw.ex_down_w.shape[1], dtype=torch.float32, device=dev)
-      C.gemm_moe(act, lw.ex_down_w, y, off, None, K.EPI["none"], T, layout_of(lw.ex_down_w) == "stream", 1, 0)
+      y = torch.empty(S * T * k, Dq, dtype=torch.float32, device=dev)
+      C.gemm_moe(act, lw.ex_down_w, y, off, None, K.EPI["none"], T, sh_dn, S, bm_dn)
     else:
       # all-fp32 run: one vendor SGEMM pair per expert that has rows (the offsets come to the host)
       y = torch.zeros(T * k, lw.ex_down_w.shape[1], dtype=torch.float32, device=dev)
@@ -606,7 +617,7 @@ class ShardModel:
       K.relu2(P, lw.ff_cols["sh_up"][0], f.shared_ff, act)
       sh_y = self._proj(act, lw.down_w)
     out = torch.empty(T, D, dtype=torch.float32, device=dev)
-    K.moe_weighted_sum(y, slot_of, topw, k, sh_y, P, lw.ff_cols["sh_gate"][0] if f.shared_ff else 0, out)
+    K.moe_weighted_sum(y, slot_of, topw, k, sh_y, P, lw.ff_cols["sh_gate"][0] if f.shared_ff else 0, out, splits=S)
     return out
 
   def _forward_postln(self, h: torch.Tensor, inp: StepInputs, adt) -> torch.Tensor:

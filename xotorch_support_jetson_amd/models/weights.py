@@ -339,6 +339,7 @@ def prepare_for_decode(sw: "ShardWeights", keep_rowmajor: Iterable[str] = (), fp
     for lw in sw.layers.values():
       if lw.in_w.dtype == torch.bfloat16:
         lw.in_w, lw.out_w, lw.down_w, lw.ff_w = wide(lw.in_w), wide(lw.out_w), wide(lw.down_w), wide(lw.ff_w)
+        lw.ex_up_w, lw.ex_down_w = conv(lw.ex_up_w), conv(lw.ex_down_w)  # experts: shuffled per expert
     if sw.lm_head is not None and sw.lm_head.dtype == torch.bfloat16:
       sw.lm_head = wide(sw.lm_head)
     return sw

@@ -557,6 +557,7 @@ def relu2(P, off: int, F: int, out) -> None:
   _mix("relu2", _gpu(P))(P, int(off), int(F), out)
 
 
-def moe_weighted_sum(y, slot_of, topw, k: int, sh_y, P, shg_off: int, out) -> None:
-  """out [T, D] fp32 = sum_j topw[t, j] * y[slot_of[t, j]] (+ sigmoid(P[t, shg_off]) * sh_y[t] for a shared expert)."""
-  _mix("moe_weighted_sum", _gpu(y))(y, slot_of, topw, int(k), sh_y, P, int(shg_off), out)
+def moe_weighted_sum(y, slot_of, topw, k: int, sh_y, P, shg_off: int, out, splits: int = 1) -> None:
+  """out [T, D] fp32 = sum_j topw[t, j] * y[slot_of[t, j]] (+ sigmoid(P[t, shg_off]) * sh_y[t] for a shared expert);
+  y [splits * T k, >= D]: the experts' down projections, K slice after K slice."""
+  _mix("moe_weighted_sum", _gpu(y))(y, slot_of, topw, int(k), sh_y, P, int(shg_off), out, int(splits))

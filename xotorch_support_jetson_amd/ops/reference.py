@@ -491,10 +491,12 @@ def relu2(P, off, Fd, out):
   out[:, :Fd] = torch.relu(P[:, off:off + Fd].float()).pow(2).to(out.dtype)
 
 
-def moe_weighted_sum(y, slot_of, topw, k, sh_y, P, shg_off, out):
-  """out [T, D] = sum_j topw[t, j] y[slot_of[t, j]] (+ sigmoid(P[t, shg_off]) sh_y[t])."""
+def moe_weighted_sum(y, slot_of, topw, k, sh_y, P, shg_off, out, splits=1):
+  """out [T, D] = sum_j topw[t, j] y[slot_of[t, j]] (+ sigmoid(P[t, shg_off]) sh_y[t]); y [splits * T k, >= D] holds
+  the down projection's K slices, summed first."""
   T, D = out.shape
-  acc = (y[slot_of.long().reshape(T, k), :D].float() * topw.reshape(T, k, 1)).sum(1)
+  y = y.reshape(splits, T * k, -1).float().sum(0)
+  acc = (y[slot_of.long().reshape(T, k), :D] * topw.reshape(T, k, 1)).sum(1)
   if sh_y is not None:
     acc = acc + torch.sigmoid(P[:, shg_off:shg_off + 1].float()) * sh_y[:, :D].float()
   out.copy_(acc)
