@@ -147,106 +147,136 @@ __global__ void kv_pool_update_k(const AT* __restrict__ k_cache, const AT* __res
 // A query at position i sees the tokens j with 0 <= i - j < window (window 0: all j <= i) and the pooled blocks b with
 // b pool + pool - 1 <= i - window; the softmax's denominator also holds exp(sink[head]).
 //
-// Workgroup per (token, head) (any d, dv <= 256, bf16 or fp32), WATT_WAVES waves: the key tiles are dealt to the waves
-// in turn; a wave's running maximum starts at -inf (wave 0: at the sink's logit with a denominator of one), lanes go
-// over keys for the scores, then over value dims for the weighted sum (token values 8 keys per 16-byte V^T load); at
-// the end the waves' (maximum, denominator, sums) are merged through LDS.
-constexpr int WATT_TILE = 256;
+// Workgroup per (token, REP query heads of one kv head) (any d, dv <= 256, bf16 or fp32), WATT_WAVES waves: the key
+// tiles are dealt to the waves in turn; a lane loads a key row once and scores it against the REP heads, and a V^T run
+// of 8 keys once for the REP weighted sums.  A wave's running maxima start at -inf (wave 0: at the sinks' logits with
+// denominators of one); at the end the waves' (maximum, denominator, sums) are merged through LDS.
 constexpr int WATT_WAVES = 8;
 
-template <typename AT>
+template <typename AT, int REP>
 __global__ __launch_bounds__(64 * WATT_WAVES) void attn_window_pool_k(
     const AT* __restrict__ q, const AT* __restrict__ k_cache, const AT* __restrict__ v_cache, const AT* __restrict__ kp,
     const AT* __restrict__ vp, const int* __restrict__ block_tables, int width, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_lens, int B, const float* __restrict__ sink, float scale, int window, int pool, int per,
     AT* __restrict__ out, int ldo, int H, int G, int d, int dv) {
+  constexpr int TILE = REP >= 8 ? 128 : 256;
   extern __shared__ float sm[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float* qs = sm;                                     // [d]
-  float* ws = sm + d + wave * WATT_TILE;              // [WATT_TILE] per wave
-  float* mg = sm + d + WATT_WAVES * WATT_TILE;        // merge: [waves][2 + dv]
-  const int t = blockIdx.x, h = blockIdx.y;
+  float* qs = sm;                                          // [REP][d]
+  float* ws = sm + REP * d + wave * REP * TILE;            // [REP][TILE] per wave
+  float* mg = sm + REP * d + WATT_WAVES * REP * TILE;      // merge: [waves][REP][2 + dv]
+  const int t = blockIdx.x, h0 = blockIdx.y * REP;
   const int b = seq_of(cu_q, B, t);
   const int ctx = ctx_lens[b];
   if (ctx <= 0) return;  // padding row of a captured decode batch
   const int pos = ctx - (cu_q[b + 1] - cu_q[b]) + (t - cu_q[b]);
-  const int g = h / (H / G);
-  for (int i = threadIdx.x; i < d; i += blockDim.x) qs[i] = ldf(q + ((int64_t)t * H + h) * d + i);
+  const int g = h0 / (H / G);
+  for (int i = threadIdx.x; i < REP * d; i += blockDim.x) qs[i] = ldf(q + ((int64_t)t * H + h0) * d + i);
   __syncthreads();
   const int* bt = block_tables + (int64_t)b * width;
-  float m = (sink && wave == 0) ? sink[h] : -INFINITY, l = (sink && wave == 0) ? 1.0f : 0.0f;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};  // value dims lane, lane + 64, ...
+  float m[REP], l[REP], acc[REP][4];  // value dims lane, lane + 64, ...
+#pragma unroll
+  for (int r = 0; r < REP; ++r) {
+    m[r] = (sink && wave == 0) ? sink[h0 + r] : -INFINITY;
+    l[r] = (sink && wave == 0) ? 1.0f : 0.0f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
+  }
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const int nbv = (pool > 0 && window > 0 && pos - window + 1 >= pool) ? (pos - window + 1) / pool : 0;
 
-  auto score = [&](const AT* kr) {
-    float s = 0.0f;
+  auto score = [&](const AT* kr, float* s) {
+#pragma unroll
+    for (int r = 0; r < REP; ++r) s[r] = 0.0f;
     if (d & 7) {
-      for (int i = 0; i < d; ++i) s += qs[i] * ldf(kr + i);
+      for (int i = 0; i < d; ++i) {
+        const float kv = ldf(kr + i);
+#pragma unroll
+        for (int r = 0; r < REP; ++r) s[r] += qs[r * d + i] * kv;
+      }
     } else {
       for (int i = 0; i < d; i += 8) {
         float kv[8];
         ld8(kr + i, kv);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) s += qs[i + e] * kv[e];
+        for (int r = 0; r < REP; ++r)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) s[r] += qs[r * d + i + e] * kv[e];
       }
     }
-    return s * scale;
+#pragma unroll
+    for (int r = 0; r < REP; ++r) s[r] *= scale;
   };
   // one tile of this wave: scores of the keys a0 + [0, n) (those outside [p0, p1) weigh nothing) -> softmax weights in
-  // ws, the running maximum / denominator / accumulators rescaled.  ws is the wave's own: its lanes' LDS accesses
+  // ws, the running maxima / denominators / accumulators rescaled.  ws is the wave's own: its lanes' LDS accesses
   // are ordered by the wave-level fences.
   auto weigh = [&](int a0, int n, int p0, int p1, auto&& key_row) {
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    float mx = -INFINITY;
-    for (int p = a0 + lane; p < a0 + n; p += 64) {
-      float s = -INFINITY;
-      if (p >= p0 && p < p1) s = score(key_row(p));
-      ws[p - a0] = s;
-      mx = fmaxf(mx, s);
-    }
-    const float mn = fmaxf(m, wave_max(mx));
-    float ls = 0.0f;
-    for (int p = a0 + lane; p < a0 + n; p += 64) {
-      const float s = ws[p - a0];
-      const float w = s == -INFINITY ? 0.0f : expf(s - mn);
-      ws[p - a0] = w;
-      ls += w;
-    }
-    const float corr = m == -INFINITY ? 0.0f : expf(m - mn);
-    l = l * corr + wave_sum(ls);
+    float mx[REP];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] *= corr;
-    m = mn;
+    for (int r = 0; r < REP; ++r) mx[r] = -INFINITY;
+    for (int p = a0 + lane; p < a0 + n; p += 64) {
+      float s[REP];
+      if (p >= p0 && p < p1) {
+        score(key_row(p), s);
+      } else {
+#pragma unroll
+        for (int r = 0; r < REP; ++r) s[r] = -INFINITY;
+      }
+#pragma unroll
+      for (int r = 0; r < REP; ++r) {
+        ws[r * TILE + p - a0] = s[r];
+        mx[r] = fmaxf(mx[r], s[r]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < REP; ++r) {
+      const float mn = fmaxf(m[r], wave_max(mx[r]));
+      float ls = 0.0f;
+      for (int p = a0 + lane; p < a0 + n; p += 64) {
+        const float s = ws[r * TILE + p - a0];
+        const float w = s == -INFINITY ? 0.0f : expf(s - mn);
+        ws[r * TILE + p - a0] = w;
+        ls += w;
+      }
+      const float corr = m[r] == -INFINITY ? 0.0f : expf(m[r] - mn);
+      l[r] = l[r] * corr + wave_sum(ls);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[r][c] *= corr;
+      m[r] = mn;
+    }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
   };
 
   int tile = 0;  // tiles are dealt to the waves in turn
   // pooled blocks [0, nbv)
-  for (int a0 = 0; a0 < nbv; a0 += WATT_TILE, ++tile) {
+  for (int a0 = 0; a0 < nbv; a0 += TILE, ++tile) {
     if (tile % WATT_WAVES != wave) continue;
-    const int n = min(WATT_TILE, nbv - a0);
+    const int n = min(TILE, nbv - a0);
     weigh(a0, n, 0, nbv, [&](int j) {
       const int pgi = (j * pool + pool - 1) / PAGE_TOK;
       return kp + (((int64_t)bt[pgi] * G + g) * per + (j - (pgi * PAGE_TOK) / pool)) * d;
     });
     for (int j = a0; j < a0 + n; ++j) {
-      const float w = ws[j - a0];
       const int pgi = (j * pool + pool - 1) / PAGE_TOK;
       const AT* vr = vp + (((int64_t)bt[pgi] * G + g) * per + (j - (pgi * PAGE_TOK) / pool)) * dv;
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         const int i = lane + 64 * c;
-        if (i < dv) acc[c] += w * ldf(vr + i);
+        if (i < dv) {
+          const float vv = ldf(vr + i);
+#pragma unroll
+          for (int r = 0; r < REP; ++r) acc[r][c] += ws[r * TILE + j - a0] * vv;
+        }
       }
     }
   }
   // tokens [lo, pos], tiles aligned to 8 keys
-  for (int a0 = lo & ~7; a0 <= pos; a0 += WATT_TILE, ++tile) {
+  for (int a0 = lo & ~7; a0 <= pos; a0 += TILE, ++tile) {
     if (tile % WATT_WAVES != wave) continue;
-    const int a1 = min(a0 + WATT_TILE, (pos + 8) & ~7);
+    const int a1 = min(a0 + TILE, (pos + 8) & ~7);
     weigh(a0, a1 - a0, lo, pos + 1, [&](int p) {
       return k_cache + (((int64_t)bt[p / PAGE_TOK] * G + g) * PAGE_TOK + (p % PAGE_TOK)) * d;
     });
@@ -259,41 +289,46 @@ __global__ __launch_bounds__(64 * WATT_WAVES) void attn_window_pool_k(
           float vv[8];
           ld8(vq + (int64_t)i * PAGE_TOK, vv);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float w = ws[p - a0 + e];
-            acc[c] += w != 0.0f ? w * vv[e] : 0.0f;  // (a slot no token has written yet may hold anything)
-          }
+          for (int r = 0; r < REP; ++r)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float w = ws[r * TILE + p - a0 + e];
+              acc[r][c] += w != 0.0f ? w * vv[e] : 0.0f;  // (a slot no token has written yet may hold anything)
+            }
         }
       }
     }
   }
   // merge the waves: M = max m_w, out = sum_w acc_w e^(m_w - M) / sum_w l_w e^(m_w - M)
-  float* mine = mg + wave * (2 + dv);
-  if (lane == 0) {
-    mine[0] = m;
-    mine[1] = l;
-  }
+  const int ms = 2 + dv;
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    const int i = lane + 64 * c;
-    if (i < dv) mine[2 + i] = acc[c];
+  for (int r = 0; r < REP; ++r) {
+    float* mine = mg + (wave * REP + r) * ms;
+    if (lane == 0) {
+      mine[0] = m[r];
+      mine[1] = l[r];
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int i = lane + 64 * c;
+      if (i < dv) mine[2 + i] = acc[r][c];
+    }
   }
   __syncthreads();
-  float M = -INFINITY;
-  for (int w = 0; w < WATT_WAVES; ++w) M = fmaxf(M, mg[w * (2 + dv)]);
-  float L = 0.0f;
-  for (int w = 0; w < WATT_WAVES; ++w) {
-    const float mw = mg[w * (2 + dv)];
-    if (mw != -INFINITY) L += mg[w * (2 + dv) + 1] * expf(mw - M);
-  }
-  const float inv = L > 0.0f ? 1.0f / L : 0.0f;
-  for (int i = threadIdx.x; i < dv; i += blockDim.x) {
-    float a = 0.0f;
+  for (int e = threadIdx.x; e < REP * dv; e += blockDim.x) {
+    const int r = e / dv, i = e - r * dv;
+    float M = -INFINITY;
+    for (int w = 0; w < WATT_WAVES; ++w) M = fmaxf(M, mg[(w * REP + r) * ms]);
+    float L = 0.0f, a = 0.0f;
     for (int w = 0; w < WATT_WAVES; ++w) {
-      const float mw = mg[w * (2 + dv)];
-      if (mw != -INFINITY) a += mg[w * (2 + dv) + 2 + i] * expf(mw - M);
+      const float* o = mg + (w * REP + r) * ms;
+      if (o[0] != -INFINITY) {
+        const float f = expf(o[0] - M);
+        L += o[1] * f;
+        a += o[2 + i] * f;
+      }
     }
-    stf(out + (int64_t)t * ldo + h * dv + i, a * inv);
+    stf(out + (int64_t)t * ldo + (h0 + r) * dv + i, L > 0.0f ? a / L : 0.0f);
   }
 }
 
@@ -827,21 +862,36 @@ void attn_window_pool(const at::Tensor& q, const at::Tensor& k_cache, const at::
                            per, out, ldo, (int)H, (int)G);
     return;
   }
-  const dim3 grid((unsigned)T, (unsigned)H);
-  const size_t lds = (size_t)(d + WATT_WAVES * WATT_TILE + WATT_WAVES * (2 + dv)) * sizeof(float);
-  if (q.scalar_type() == at::kBFloat16)
-    attn_window_pool_k<uint16_t><<<grid, 64 * WATT_WAVES, lds, stream()>>>(
-        (const uint16_t*)q.data_ptr(), (const uint16_t*)k_cache.data_ptr(), (const uint16_t*)v_cache.data_ptr(),
-        pooled ? (const uint16_t*)kp->data_ptr() : nullptr, pooled ? (const uint16_t*)vp->data_ptr() : nullptr,
-        block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, sp,
-        (float)scale, (int)window, pooled ? (int)pool : 0, per, (uint16_t*)out.data_ptr(), ldo, (int)H, (int)G, (int)d,
-        (int)dv);
-  else
-    attn_window_pool_k<float><<<grid, 64 * WATT_WAVES, lds, stream()>>>(
-        q.data_ptr<float>(), k_cache.data_ptr<float>(), v_cache.data_ptr<float>(),
-        pooled ? kp->data_ptr<float>() : nullptr, pooled ? vp->data_ptr<float>() : nullptr, block_tables.data_ptr<int>(),
-        (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, sp, (float)scale, (int)window,
-        pooled ? (int)pool : 0, per, out.data_ptr<float>(), ldo, (int)H, (int)G, (int)d, (int)dv);
+  // query heads of one kv head share a workgroup (each key row and value run is loaded once for all of them)
+  const int rep_all = (int)(H / G);
+  int rep = rep_all % 8 == 0 ? 8 : rep_all % 4 == 0 ? 4 : rep_all % 2 == 0 ? 2 : 1;
+  auto lds_of = [&](int r) {
+    return (size_t)(r * d + WATT_WAVES * r * (r >= 8 ? 128 : 256) + WATT_WAVES * r * (2 + dv)) * sizeof(float);
+  };
+  // (the default limit of dynamic LDS per workgroup is 64 KB; a small step keeps a workgroup per head to fill the chip)
+  while (rep > 1 && (lds_of(rep) > 60 * 1024 || T * (H / rep) < 256)) rep /= 2;
+  const dim3 grid((unsigned)T, (unsigned)(H / rep));
+  const size_t lds = lds_of(rep);
+#define WATT_GO(AT, R)                                                                                                     \
+  attn_window_pool_k<AT, R><<<grid, 64 * WATT_WAVES, lds, stream()>>>(                                                     \
+      (const AT*)q.data_ptr(), (const AT*)k_cache.data_ptr(), (const AT*)v_cache.data_ptr(),                               \
+      pooled ? (const AT*)kp->data_ptr() : nullptr, pooled ? (const AT*)vp->data_ptr() : nullptr,                          \
+      block_tables.data_ptr<int>(), (int)block_tables.size(1), cu_q.data_ptr<int>(), ctx_lens.data_ptr<int>(), (int)B, sp, \
+      (float)scale, (int)window, pooled ? (int)pool : 0, per, (AT*)out.data_ptr(), ldo, (int)H, (int)G, (int)d, (int)dv)
+#define WATT_REP(AT)                   \
+  switch (rep) {                       \
+    case 8: WATT_GO(AT, 8); break;     \
+    case 4: WATT_GO(AT, 4); break;     \
+    case 2: WATT_GO(AT, 2); break;     \
+    default: WATT_GO(AT, 1); break;    \
+  }
+  if (q.scalar_type() == at::kBFloat16) {
+    WATT_REP(uint16_t)
+  } else {
+    WATT_REP(float)
+  }
+#undef WATT_REP
+#undef WATT_GO
 }
 
 void ssd_prep(const at::Tensor& P, int64_t x_off, int64_t dt_off, const at::Tensor& conv_w, const at::Tensor& conv_b,
