@@ -685,10 +685,10 @@ TINY_MOGELIX = {
     {"type": "mamba2", "mlp": {"kind": "dense", "ff": 160},
      "mixer": {"heads": 4, "vdim": 16, "state": 24, "groups": 2, "conv": 3, "norm_groups": 2}},
     {"type": "attention", "mlp": _TINY_MOE,
-     "mixer": {"heads": 6, "kv_heads": 2, "dim": 32, "vdim": 16, "mask": {"size": 20, "pool": 5}, "rot": _TINY_ROT,
+     "mixer": {"heads": 6, "kv_heads": 2, "dim": 16, "vdim": 32, "mask": {"size": 20, "pool": 5}, "rot": _TINY_ROT,
                "scale": 0.3}},
     {"type": "attention", "mlp": None,
-     "mixer": {"heads": 6, "kv_heads": 2, "dim": 32, "vdim": 16, "kv_from": 1, "mask": {"size": 9, "pool": 3},
+     "mixer": {"heads": 6, "kv_heads": 2, "dim": 16, "vdim": 32, "kv_from": 1, "mask": {"size": 9, "pool": 3},
                "rot": _TINY_ROT, "scale": 0.25}},
     {"type": "mamba2", "mlp": _TINY_MOE,
      "mixer": {"heads": 2, "vdim": 32, "state": 16, "groups": 1, "conv": 4, "norm_groups": 1}},
