@@ -244,6 +244,9 @@ SIZES = [
   config([layer("attention", attn(4, 2, 16, 8, 12, 4), dense(32)), layer("attention", attn(4, 2, 16, 8, 12, 4, kv_from=0), None),
           layer("mamba2", ssd(2, 8, 8, 2, 5, 1), None), layer("attention", attn(2, 2, 16, 8, 30, 8, kv_from=0), moe(8, 7, 3, 8)),
           layer("attention", attn(2, 2, 16, 8, 0, 0, kv_from=0), None)], width=40),
+  # more experts and more chosen than the small routing kernel takes
+  config([layer("mamba2", ssd(2, 8, 8, 1, 2, 1), moe(8, 70, 9, 0)), layer("attention", attn(2, 1, 16, 16, 6, 2), moe(8, 3, 2, 8))],
+         width=32, vocab=40),
 ]
 
 
