@@ -558,6 +558,9 @@ __global__ void ssd_prep_k(const float* __restrict__ P, int ldp, int x_off, int 
   const float* row = P + (int64_t)t * ldp;
   const float* st = conv_state + (int64_t)slot * (taps - 1) * C;
   const int inner = H * dv;
+  extern __shared__ float dts[];  // [H] step sizes of this token
+  for (int h = threadIdx.x; h < H; h += blockDim.x) dts[h] = softplusf_(row[dt_off + h] + dt_bias[h]);
+  __syncthreads();
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
     float acc = conv_b[c];
     for (int j = 0; j < taps; ++j) {
@@ -567,14 +570,10 @@ __global__ void ssd_prep_k(const float* __restrict__ P, int ldp, int x_off, int 
     }
     const float y = siluf_(acc);
     xbc[(int64_t)t * C + c] = y;
-    if (c < inner) {
-      const int h = c / dv;
-      v[(int64_t)t * inner + c] = softplusf_(row[dt_off + h] + dt_bias[h]) * y;
-    }
+    if (c < inner) v[(int64_t)t * inner + c] = dts[c / dv] * y;
   }
   if (blockIdx.y == 0)
-    for (int h = threadIdx.x; h < H; h += blockDim.x)
-      decay[(int64_t)t * H + h] = expf(-expf(A_log[h]) * softplusf_(row[dt_off + h] + dt_bias[h]));
+    for (int h = threadIdx.x; h < H; h += blockDim.x) decay[(int64_t)t * H + h] = expf(-expf(A_log[h]) * dts[h]);
 }
 
 // the last taps - 1 convolution inputs of every sequence -> its state slot (after every token of the step has read
@@ -620,27 +619,54 @@ __global__ void ssd_gate_norm_k(const float* __restrict__ o, const float* __rest
 }
 
 // ------------------------------------------------------------------ PolyNorm
+// One workgroup per token.  Rows of at most PN_REG values a thread are read once and kept in registers between the
+// three sums and the polynomial; longer rows are read twice.
+constexpr int PN_REG = 16;
+
 template <typename AT>
 __global__ void polynorm_act_k(const float* __restrict__ P, int ldp, int up_off, int F, const float* __restrict__ coef,
                                float eps, AT* __restrict__ out, int ldo) {
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
   const float* z = P + t * ldp + up_off;
+  const bool held = F <= PN_REG * (int)blockDim.x;
+  float zr[PN_REG];
   float s2 = 0.0f, s4 = 0.0f, s6 = 0.0f;
-  for (int i = threadIdx.x; i < F; i += blockDim.x) {
-    const float a = z[i], a2 = a * a, a3 = a2 * a;
-    s2 += a2;
-    s4 += a2 * a2;
-    s6 += a3 * a3;
+  if (held) {
+#pragma unroll
+    for (int j = 0; j < PN_REG; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      const float a = i < F ? z[i] : 0.0f, a2 = a * a, a3 = a2 * a;
+      zr[j] = a;
+      s2 += a2;
+      s4 += a2 * a2;
+      s6 += a3 * a3;
+    }
+  } else {
+    for (int i = threadIdx.x; i < F; i += blockDim.x) {
+      const float a = z[i], a2 = a * a, a3 = a2 * a;
+      s2 += a2;
+      s4 += a2 * a2;
+      s6 += a3 * a3;
+    }
   }
   s2 = block_sum(s2, red);
   s4 = block_sum(s4, red);
   s6 = block_sum(s6, red);
   const float k1 = coef[0] / sqrtf(s2 / (float)F + eps), k2 = coef[1] / sqrtf(s4 / (float)F + eps),
               k3 = coef[2] / sqrtf(s6 / (float)F + eps), e = coef[3];
-  for (int i = threadIdx.x; i < F; i += blockDim.x) {
-    const float a = z[i], a2 = a * a;
-    stf(out + t * ldo + i, k1 * a + k2 * a2 + k3 * a2 * a + e);
+  if (held) {
+#pragma unroll
+    for (int j = 0; j < PN_REG; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      const float a = zr[j], a2 = a * a;
+      if (i < F) stf(out + t * ldo + i, k1 * a + k2 * a2 + k3 * a2 * a + e);
+    }
+  } else {
+    for (int i = threadIdx.x; i < F; i += blockDim.x) {
+      const float a = z[i], a2 = a * a;
+      stf(out + t * ldo + i, k1 * a + k2 * a2 + k3 * a2 * a + e);
+    }
   }
 }
 
@@ -921,7 +947,7 @@ void ssd_prep(const at::Tensor& P, int64_t x_off, int64_t dt_off, const at::Tens
   cols_ok(P, dt_off, H, "dt");
   // few tokens (decode steps): the channels are spread over workgroups too
   const dim3 pgrid((unsigned)T, (unsigned)(T >= 2048 ? 1 : std::min<int64_t>((C + 255) / 256, 32)));
-  ssd_prep_k<<<pgrid, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)x_off, (int)dt_off, conv_w.data_ptr<float>(),
+  ssd_prep_k<<<pgrid, 256, H * sizeof(float), stream()>>>(P.data_ptr<float>(), ldp, (int)x_off, (int)dt_off, conv_w.data_ptr<float>(),
                                       conv_b.data_ptr<float>(), (int)taps, (int)C, conv_state.data_ptr<float>(),
                                       state_slots.data_ptr<int>(), cu_q.data_ptr<int>(), (int)B, A_log.data_ptr<float>(),
                                       dt_bias.data_ptr<float>(), (int)H, (int)dv, xbc.data_ptr<float>(), v.data_ptr<float>(),
@@ -970,12 +996,13 @@ void polynorm_act(const at::Tensor& P, int64_t up_off, int64_t F, const at::Tens
   MCHECK(coef.numel() == 4 && F > 0, "PolyNorm takes four coefficients");
   cols_ok(P, up_off, F, "up");
   const int ldo = act_ld_min(out, T, F, "out");
+  const int bs = F > 256 * PN_REG ? 1024 : 256;
   if (out.scalar_type() == at::kBFloat16)
-    polynorm_act_k<uint16_t><<<T, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)up_off, (int)F, coef.data_ptr<float>(),
-                                                      (float)eps, (uint16_t*)out.data_ptr(), ldo);
+    polynorm_act_k<uint16_t><<<T, bs, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)up_off, (int)F, coef.data_ptr<float>(),
+                                                     (float)eps, (uint16_t*)out.data_ptr(), ldo);
   else
-    polynorm_act_k<float><<<T, 256, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)up_off, (int)F, coef.data_ptr<float>(),
-                                                   (float)eps, out.data_ptr<float>(), ldo);
+    polynorm_act_k<float><<<T, bs, 0, stream()>>>(P.data_ptr<float>(), ldp, (int)up_off, (int)F, coef.data_ptr<float>(),
+                                                  (float)eps, out.data_ptr<float>(), ldo);
 }
 
 void relu2(const at::Tensor& P, int64_t off, int64_t F, at::Tensor& out) {
